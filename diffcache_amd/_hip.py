@@ -1,0 +1,340 @@
+"""ctypes binding of ``libdiffcache_hip.so`` and tensor-level wrappers.
+
+The library is the product; there is no CPU or PyTorch fallback.  Importing
+this module without the built library raises, and every wrapper raises if a
+tensor is not on a GPU.  PyTorch is used only for device memory and streams.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+import os
+from typing import Optional, Tuple
+
+import torch
+
+MODE_IP = 0
+MODE_REF_DIST = 1
+ORDER_ANY = 0
+ORDER_BEST = 1
+ORDER_INDEX = 2
+HIST_BINS = 4096
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdiffcache_hip.so")
+
+# every symbol include/diffcache_hip.h declares
+SYMBOLS = (
+    "dc_version", "dc_last_error", "dc_group_mean_bf16", "dc_score_bf16",
+    "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
+    "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_append_kv_bf16",
+    "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
+    "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
+)
+
+
+class LayerArgs(C.Structure):
+    """struct dc_layer_args of include/diffcache_hip.h"""
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+        ("new_k", C.c_void_p), ("new_v", C.c_void_p), ("out", C.c_void_p),
+        ("lse", C.c_void_p), ("scores", C.c_void_p), ("idx_out", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("kv_batch_stride", C.c_int64), ("kv_head_stride", C.c_int64), ("kv_row_stride", C.c_int64),
+        ("scores_unit_stride", C.c_int64), ("idx_unit_stride", C.c_int64),
+        ("recent_lo", C.c_int64),
+        ("n_b", C.c_int), ("n_h", C.c_int), ("group", C.c_int), ("hd", C.c_int),
+        ("n_sink", C.c_int), ("n_recent", C.c_int), ("budget", C.c_int),
+        ("mode", C.c_int), ("order", C.c_int), ("scale", C.c_float),
+    ]
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m diffcache_amd.build` "
+            "(hipcc, --offload-arch=gfx950). There is no fallback path.")
+    lib = C.CDLL(LIB_PATH)
+    i, i64, p, sz, f = C.c_int, C.c_int64, C.c_void_p, C.c_size_t, C.c_float
+    sigs = {
+        "dc_version": (i, []),
+        "dc_last_error": (C.c_char_p, []),
+        "dc_group_mean_bf16": (i, [p, p, i, i, i, p]),
+        "dc_score_bf16": (i, [p, p, p, p, i, i, i, i, i64, i64, i64, i64, i, i, p]),
+        "dc_topk_workspace_bytes": (sz, [i, i, i]),
+        "dc_topk_select": (i, [p, i64, p, i64, i, i, i, i, i, p, p, sz, p]),
+        "dc_gather_rows_bf16": (i, [p, p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, i64, i64, p]),
+        "dc_attn_workspace_bytes": (sz, [i, i, i, i]),
+        "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i, i64, i,
+                                    i64, i64, i64, i64, i64, i64, f, p, sz, p]),
+        "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, i64, i64, i64, p]),
+        "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
+        "dc_layer_workspace_bytes": (sz, [i, i, i, i, i, i]),
+        "dc_decode_layer": (i, [C.POINTER(LayerArgs), p]),
+        "dc_pq_build_lut": (i, [p, p, p, i, i, i, i, p]),
+        "dc_pq_adc_scan": (i, [p, p, p, p, i, i, i, i64, p]),
+        "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
+        "dc_compose_idx": (i, [p, i64, p, i64, p, i64, i, i, p]),
+    }
+    for name, (res, args) in sigs.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+class DiffCacheError(RuntimeError):
+    pass
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise DiffCacheError(f"[{rc}] {lib.dc_last_error().decode()}")
+
+
+def _dev(t: torch.Tensor, name: str) -> int:
+    if not t.is_cuda:
+        raise DiffCacheError(f"{name} must live in GPU memory (got {t.device}); there is no CPU path")
+    return t.data_ptr()
+
+
+def _opt(t: Optional[torch.Tensor], name: str):
+    return None if t is None else _dev(t, name)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _store_strides(store: torch.Tensor) -> Tuple[int, int, int]:
+    """(batch, head, row) element strides of a (b, h, n, hd) bf16 store."""
+    if store.dim() != 4 or store.dtype != torch.bfloat16 or store.stride(3) != 1:
+        raise DiffCacheError("a K/V store must be a (b, h, n, hd) bfloat16 tensor with contiguous rows")
+    return store.stride(0), store.stride(1), store.stride(2)
+
+
+def alloc_workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty((max(int(nbytes), 256) + 255) // 256 * 256, dtype=torch.uint8, device=device)
+
+
+# ---------------------------------------------------------------------------
+# wrappers
+# ---------------------------------------------------------------------------
+
+def group_mean(q: torch.Tensor, group: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q (..., group, hd) bf16 viewed as (n_units, group, hd) -> (n_units, hd) bf16."""
+    hd = q.shape[-1]
+    q = q.contiguous()
+    n_units = q.numel() // (group * hd)
+    if out is None:
+        out = torch.empty((n_units, hd), dtype=torch.bfloat16, device=q.device)
+    _check(lib.dc_group_mean_bf16(_dev(q, "q"), _dev(out, "out"), n_units, group, hd, _stream()))
+    return out
+
+
+def score(store_k: torch.Tensor, q: torch.Tensor, lo: int, n_rows: int, mode: int = MODE_REF_DIST,
+          q_group: int = 1, scores: Optional[torch.Tensor] = None,
+          hist: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Scores of rows [lo, lo + n_rows) of every unit.  q: (b*h*q_group*hd) bf16 in
+    (b, h, q_group, hd) order.  Returns fp32 (b*h, n_rows)."""
+    sb, sh, sr = _store_strides(store_k)
+    b, h, n_max, hd = store_k.shape
+    if lo < 0 or lo + n_rows > n_max:
+        raise DiffCacheError(f"rows [{lo}, {lo + n_rows}) outside the store of {n_max} rows")
+    q = q.contiguous()
+    if q.dtype != torch.bfloat16 or q.numel() != b * h * q_group * hd:
+        raise DiffCacheError("q must be bf16 with b*h*q_group*hd elements")
+    if scores is None:
+        scores = torch.empty((b * h, n_rows), dtype=torch.float32, device=store_k.device)
+    kptr = _dev(store_k, "store_k") + lo * sr * 2
+    _check(lib.dc_score_bf16(kptr, _dev(q, "q"), _dev(scores, "scores"), _opt(hist, "hist"), b, h,
+                             n_rows, hd, sb, sh, sr, scores.stride(0), q_group, mode, _stream()))
+    return scores
+
+
+def new_hist(n_units: int, device) -> torch.Tensor:
+    return torch.zeros((n_units, HIST_BINS), dtype=torch.int32, device=device)
+
+
+def topk_select(scores: torch.Tensor, k: int, mode: int = MODE_REF_DIST, order: int = ORDER_ANY,
+                hist: Optional[torch.Tensor] = None, idx_out: Optional[torch.Tensor] = None,
+                workspace: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
+    """scores (n_units, >= n_rows) fp32 -> int32 ids (n_units, min(k, n_rows))."""
+    if scores.dim() != 2 or scores.dtype != torch.float32 or scores.stride(1) != 1:
+        raise DiffCacheError("scores must be a (n_units, n_rows) fp32 tensor with contiguous rows")
+    n_units = scores.shape[0]
+    n_rows = scores.shape[1] if n_rows is None else n_rows
+    k_eff = min(k, n_rows)
+    if idx_out is None:
+        idx_out = torch.empty((n_units, max(k_eff, 1)), dtype=torch.int32, device=scores.device)
+    need = lib.dc_topk_workspace_bytes(n_units, n_rows, k)
+    if workspace is None:
+        workspace = alloc_workspace(need, scores.device)
+    _check(lib.dc_topk_select(_dev(scores, "scores"), scores.stride(0), _dev(idx_out, "idx_out"),
+                              idx_out.stride(0), n_units, n_rows, k, mode, order, _opt(hist, "hist"),
+                              _dev(workspace, "workspace"), workspace.numel(), _stream()))
+    return idx_out[:, :k_eff]
+
+
+def gather_rows(store_k: Optional[torch.Tensor], store_v: Optional[torch.Tensor], idx: torch.Tensor,
+                out_k: Optional[torch.Tensor], out_v: Optional[torch.Tensor], row_offset: int = 0,
+                n_idx: Optional[int] = None) -> None:
+    """out[b, h, j, :] = store[b, h, row_offset + idx[b*H + h, j], :] for j < n_idx."""
+    ref = store_k if store_k is not None else store_v
+    sb, sh, sr = _store_strides(ref)
+    b, h, _, hd = ref.shape
+    dst = out_k if out_k is not None else out_v
+    db, dh, dr = _store_strides(dst)
+    n_idx = idx.shape[1] if n_idx is None else n_idx
+    _check(lib.dc_gather_rows_bf16(_opt(store_k, "store_k"), _opt(store_v, "store_v"), _dev(idx, "idx"),
+                                   _opt(out_k, "out_k"), _opt(out_v, "out_v"), b, h, n_idx,
+                                   idx.stride(0), hd, row_offset, sb, sh, sr, db, dh, dr, _stream()))
+
+
+def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
+                idx: Optional[torch.Tensor], n_idx: int, region_lo: int, n_sink: int, recent_lo: int,
+                n_recent: int, new_k: Optional[torch.Tensor] = None,
+                new_v: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q (b, h*group, hd) bf16 -> out (b, h*group, hd) bf16."""
+    ksb, ksh, ksr = _store_strides(store_k)
+    vsb, vsh, vsr = _store_strides(store_v)
+    b, h, _, hd = store_k.shape
+    q = q.contiguous()
+    group = q.numel() // (b * h * hd)
+    if out is None:
+        out = torch.empty((b, h * group, hd), dtype=torch.bfloat16, device=q.device)
+    scale = 1.0 / math.sqrt(hd) if scale is None else scale
+    n_total = n_idx + n_sink + n_recent + (1 if new_k is not None else 0)
+    need = lib.dc_attn_workspace_bytes(b * h, group, hd, n_total)
+    if workspace is None:
+        workspace = alloc_workspace(need, q.device)
+    if new_k is not None:
+        new_k, new_v = new_k.contiguous(), new_v.contiguous()
+    _check(lib.dc_gather_attn_bf16(
+        _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v"), _opt(idx, "idx"),
+        _opt(new_k, "new_k"), _opt(new_v, "new_v"), _dev(out, "out"), _opt(lse, "lse"), b, h, group,
+        hd, n_idx, 0 if idx is None else idx.stride(0), region_lo, n_sink, recent_lo, n_recent,
+        ksb, ksh, ksr, vsb, vsh, vsr, scale, _dev(workspace, "workspace"), workspace.numel(),
+        _stream()))
+    return out
+
+
+def append_kv(store_k: torch.Tensor, store_v: torch.Tensor, new_k: torch.Tensor,
+              new_v: torch.Tensor, pos: int) -> None:
+    sb, sh, sr = _store_strides(store_k)
+    if _store_strides(store_v) != (sb, sh, sr):
+        raise DiffCacheError("K and V stores must share their strides")
+    b, h, n_max, hd = store_k.shape
+    if not 0 <= pos < n_max:
+        raise DiffCacheError(f"append position {pos} outside the store of {n_max} rows")
+    new_k, new_v = new_k.contiguous(), new_v.contiguous()
+    if new_k.numel() != b * h * hd or new_v.numel() != b * h * hd:
+        raise DiffCacheError("new_k/new_v must hold (b, h, hd) values")
+    _check(lib.dc_append_kv_bf16(_dev(store_k, "store_k"), _dev(store_v, "store_v"),
+                                 _dev(new_k, "new_k"), _dev(new_v, "new_v"), b, h, hd, pos, sb, sh, sr,
+                                 _stream()))
+
+
+def ingest_kv(store: torch.Tensor, src: torch.Tensor, dst_pos: int = 0) -> None:
+    """src (b, seq, h, hd) bf16 -> store[b, h, dst_pos + s, :]."""
+    sb, sh, sr = _store_strides(store)
+    b, h, n_max, hd = store.shape
+    src = src.contiguous()
+    if src.dtype != torch.bfloat16 or src.dim() != 4 or src.shape[0] != b or src.shape[2] != h \
+            or src.shape[3] != hd:
+        raise DiffCacheError("src must be a (b, seq, h, hd) bf16 tensor matching the store")
+    seq = src.shape[1]
+    if dst_pos < 0 or dst_pos + seq > n_max:
+        raise DiffCacheError(f"rows [{dst_pos}, {dst_pos + seq}) outside the store of {n_max} rows")
+    _check(lib.dc_ingest_kv_bf16(_dev(store, "store"), _dev(src, "src"), b, seq, h, hd, dst_pos, sb, sh,
+                                 sr, _stream()))
+
+
+def layer_workspace_bytes(n_units: int, n_region: int, budget: int, group: int, hd: int,
+                          n_attended: int) -> int:
+    return int(lib.dc_layer_workspace_bytes(n_units, n_region, budget, group, hd, n_attended))
+
+
+def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, n_sink: int,
+                 recent_lo: int, n_recent: int, budget: int, scores: torch.Tensor,
+                 idx_out: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor,
+                 new_k: Optional[torch.Tensor] = None, new_v: Optional[torch.Tensor] = None,
+                 lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
+                 order: int = ORDER_ANY, scale: Optional[float] = None) -> torch.Tensor:
+    """score -> select -> attend for one layer, enqueued on the current stream."""
+    sb, sh, sr = _store_strides(store_k)
+    if _store_strides(store_v) != (sb, sh, sr):
+        raise DiffCacheError("K and V stores must share their strides")
+    b, h, n_max, hd = store_k.shape
+    if recent_lo + n_recent > n_max:
+        raise DiffCacheError("recent window runs past the end of the store")
+    if not q.is_contiguous():
+        raise DiffCacheError("q must be contiguous")
+    group = q.numel() // (b * h * hd)
+    a = LayerArgs()
+    a.q, a.k, a.v = _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v")
+    a.new_k, a.new_v = _opt(new_k, "new_k"), _opt(new_v, "new_v")
+    a.out, a.lse = _dev(out, "out"), _opt(lse, "lse")
+    a.scores, a.idx_out = _dev(scores, "scores"), _dev(idx_out, "idx_out")
+    a.workspace, a.workspace_bytes = _dev(workspace, "workspace"), workspace.numel()
+    a.kv_batch_stride, a.kv_head_stride, a.kv_row_stride = sb, sh, sr
+    a.scores_unit_stride, a.idx_unit_stride = scores.stride(0), idx_out.stride(0)
+    a.recent_lo = recent_lo
+    a.n_b, a.n_h, a.group, a.hd = b, h, group, hd
+    a.n_sink, a.n_recent, a.budget = n_sink, n_recent, budget
+    a.mode, a.order = mode, order
+    a.scale = 1.0 / math.sqrt(hd) if scale is None else scale
+    _check(lib.dc_decode_layer(C.byref(a), _stream()))
+    return out
+
+
+# ---- PQ baseline ----
+
+def pq_build_lut(q: torch.Tensor, books: torch.Tensor, n_b: int) -> torch.Tensor:
+    """q (n_b*n_h, hd) bf16, books (n_h, M, 256, ds) fp32 -> lut (n_b*n_h, M, 256) fp32."""
+    n_h, m, nc, ds = books.shape
+    if nc != 256 or books.dtype != torch.float32:
+        raise DiffCacheError("books must be (n_h, M, 256, ds) fp32")
+    q, books = q.contiguous(), books.contiguous()
+    lut = torch.empty((n_b * n_h, m, 256), dtype=torch.float32, device=q.device)
+    _check(lib.dc_pq_build_lut(_dev(q, "q"), _dev(books, "books"), _dev(lut, "lut"), n_b, n_h, m * ds, m,
+                               _stream()))
+    return lut
+
+
+def pq_adc_scan(codes: torch.Tensor, lut: torch.Tensor, hist: Optional[torch.Tensor] = None
+                ) -> torch.Tensor:
+    """codes (n_units, n_rows, M) uint8, lut (n_units, M, 256) -> scores (n_units, n_rows) fp32."""
+    n_units, n_rows, m = codes.shape
+    codes, lut = codes.contiguous(), lut.contiguous()
+    scores = torch.empty((n_units, n_rows), dtype=torch.float32, device=codes.device)
+    _check(lib.dc_pq_adc_scan(_dev(codes, "codes"), _dev(lut, "lut"), _dev(scores, "scores"),
+                              _opt(hist, "hist"), n_units, n_rows, m, scores.stride(0), _stream()))
+    return scores
+
+
+def score_gathered(store_k: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, row_offset: int = 0
+                   ) -> torch.Tensor:
+    sb, sh, sr = _store_strides(store_k)
+    b, h, _, hd = store_k.shape
+    q = q.contiguous()
+    n_idx = idx.shape[1]
+    scores = torch.empty((b * h, n_idx), dtype=torch.float32, device=q.device)
+    _check(lib.dc_score_gathered_bf16(_dev(store_k, "store_k"), _dev(q, "q"), _dev(idx, "idx"),
+                                      _dev(scores, "scores"), b, h, n_idx, idx.stride(0), hd, row_offset,
+                                      sb, sh, sr, scores.stride(0), _stream()))
+    return scores
+
+
+def compose_idx(outer: torch.Tensor, inner: torch.Tensor) -> torch.Tensor:
+    n_units, n_inner = inner.shape
+    out = torch.empty((n_units, n_inner), dtype=torch.int32, device=inner.device)
+    _check(lib.dc_compose_idx(_dev(outer, "outer"), outer.stride(0), _dev(inner, "inner"),
+                              inner.stride(0), _dev(out, "out"), out.stride(0), n_units, n_inner,
+                              _stream()))
+    return out

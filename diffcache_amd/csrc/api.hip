@@ -1,0 +1,105 @@
+// Error plumbing, version, and the fused per-layer call chain of the C ABI.
+#include "dc_common.h"
+#include <stdarg.h>
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+void dc_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" int dc_version(void) { return DC_VERSION; }
+
+extern "C" const char *dc_last_error(void) { return g_err; }
+
+namespace {
+
+__global__ void fill_zero_kernel(uint32_t *p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+struct LayerWs {
+    uint32_t *hist;
+    void *topk;
+    size_t topk_bytes;
+    void *attn;
+    size_t attn_bytes;
+    size_t bytes;
+};
+
+LayerWs carve_layer(void *base, int n_units, int n_region, int budget, int group, int hd,
+                    int n_attended) {
+    LayerWs w;
+    char *p = (char *)base;
+    size_t off = 0;
+    w.hist = (uint32_t *)(p + off);
+    off += dc_align_up((size_t)(n_units > 0 ? n_units : 0) * DC_HIST_BINS * 4, 256);
+    w.topk = p + off;
+    w.topk_bytes = dc_align_up(dc_topk_workspace_bytes(n_units, n_region, budget), 256);
+    off += w.topk_bytes;
+    w.attn = p + off;
+    w.attn_bytes = dc_align_up(dc_attn_workspace_bytes(n_units, group, hd, n_attended), 256);
+    off += w.attn_bytes;
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group,
+                                           int hd, int n_rows_attended) {
+    return carve_layer(nullptr, n_units, n_region_rows, budget, group, hd, n_rows_attended).bytes;
+}
+
+extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
+    DC_REQUIRE(a, "dc_decode_layer: null args");
+    DC_REQUIRE(a->q && a->k && a->v && a->out && a->scores && a->idx_out,
+               "dc_decode_layer: null pointer in args");
+    DC_REQUIRE(a->n_b >= 0 && a->n_h >= 1 && a->group >= 1 && a->n_sink >= 0 && a->n_recent >= 0 &&
+                   a->budget >= 0,
+               "dc_decode_layer: bad sizes");
+    DC_REQUIRE(a->recent_lo >= a->n_sink, "dc_decode_layer: recent_lo %lld < n_sink %d",
+               (long long)a->recent_lo, a->n_sink);
+    const int n_units = a->n_b * a->n_h;
+    if (n_units == 0) return DC_OK;
+    const int64_t region64 = a->recent_lo - a->n_sink;
+    DC_REQUIRE(region64 < (1ll << 31), "dc_decode_layer: region too long");
+    const int region = (int)region64;
+    const int k_eff = a->budget < region ? a->budget : region;
+    const int has_new = a->new_k ? 1 : 0;
+    const int attended = k_eff + a->n_sink + a->n_recent + has_new;
+    DC_REQUIRE(a->workspace && (((uintptr_t)a->workspace) & 255u) == 0,
+               "dc_decode_layer: workspace must be non-null and 256-byte aligned");
+    LayerWs w = carve_layer(a->workspace, n_units, region, a->budget, a->group, a->hd, attended);
+    if (a->workspace_bytes < w.bytes) {
+        dc_set_error("dc_decode_layer: workspace %zu bytes < %zu needed", a->workspace_bytes, w.bytes);
+        return DC_ENOMEM;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    int rc;
+    if (k_eff > 0) {
+        const int64_t n = (int64_t)n_units * DC_HIST_BINS;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                           w.hist, n);
+        DC_CHECK_LAUNCH("dc_decode_layer(zero)");
+        const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
+        rc = dc_score_bf16(k_region, a->q, a->scores, w.hist, a->n_b, a->n_h, region, a->hd,
+                           a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride,
+                           a->scores_unit_stride, a->group, a->mode, stream);
+        if (rc) return rc;
+        rc = dc_topk_select(a->scores, a->scores_unit_stride, a->idx_out, a->idx_unit_stride, n_units,
+                            region, a->budget, a->mode, a->order, w.hist, w.topk, w.topk_bytes, stream);
+        if (rc) return rc;
+    }
+    rc = dc_gather_attn_bf16(a->q, a->k, a->v, a->idx_out, a->new_k, a->new_v, a->out, a->lse, a->n_b,
+                             a->n_h, a->group, a->hd, k_eff, a->idx_unit_stride, a->n_sink, a->n_sink,
+                             a->recent_lo, a->n_recent, a->kv_batch_stride, a->kv_head_stride,
+                             a->kv_row_stride, a->kv_batch_stride, a->kv_head_stride,
+                             a->kv_row_stride, a->scale, w.attn, w.attn_bytes, stream);
+    return rc;
+}

@@ -1,0 +1,107 @@
+// Shared device helpers and host-side error plumbing for libdiffcache_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/diffcache_hip.h"
+
+#define DC_WAVE 64
+
+// ---- host side -------------------------------------------------------------
+void dc_set_error(const char *fmt, ...);
+
+#define DC_REQUIRE(cond, ...)            \
+    do {                                 \
+        if (!(cond)) {                   \
+            dc_set_error(__VA_ARGS__);   \
+            return DC_EINVAL;            \
+        }                                \
+    } while (0)
+
+#define DC_CHECK_LAUNCH(name)                                              \
+    do {                                                                   \
+        hipError_t e_ = hipGetLastError();                                 \
+        if (e_ != hipSuccess) {                                            \
+            dc_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+            return DC_ELAUNCH;                                             \
+        }                                                                  \
+    } while (0)
+
+static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---- device side -----------------------------------------------------------
+__device__ __forceinline__ float dc_bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float dc_bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float dc_bf16_to_f32(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round to nearest even; NaN -> canonical quiet NaN
+__device__ __forceinline__ uint16_t dc_f32_to_bf16(float f) {
+    uint32_t b = __float_as_uint(f);
+    if ((b & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    uint32_t lsb = (b >> 16) & 1u;
+    return (uint16_t)((b + 0x7fffu + lsb) >> 16);
+}
+
+// order-preserving map f32 -> u32 (ascending)
+__device__ __forceinline__ uint32_t dc_f2ord(float x) {
+    uint32_t b = __float_as_uint(x);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// 32-bit ordering key (smaller = better) and its coarse histogram bucket.
+// The bucket is a monotone function of the key, so equal keys share a bucket.
+// DC_MODE_IP:       key = ord(-(s + 0)),            bucket = key >> 20
+// DC_MODE_REF_DIST: key = ord(d), d = f32(65536-s); bucket from s' = 65536 - d,
+//                   which is exact and is s rounded onto d's grid.
+__device__ __forceinline__ void dc_key_bucket(float s, int mode, uint32_t &key, uint32_t &bucket) {
+    if (mode == DC_MODE_REF_DIST) {
+        float d = 65536.0f - s;
+        key = dc_f2ord(d);
+        float sq = 65536.0f - d;
+        bucket = dc_f2ord(-(sq + 0.0f)) >> 20;
+    } else {
+        key = dc_f2ord(-(s + 0.0f));
+        bucket = key >> 20;
+    }
+}
+
+// sum over the 16 lanes of a DPP row; every lane of the row receives the sum
+__device__ __forceinline__ float dc_row16_sum(float v) {
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0x140, 0xF, 0xF, true);  // row_mirror
+    return v;
+}
+
+// sum over aligned groups of 8 lanes
+__device__ __forceinline__ float dc_row8_sum(float v) {
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0xB1, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0x4E, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0.0f, v, 0x141, 0xF, 0xF, true);
+    return v;
+}
+
+// sum over aligned groups of LPR lanes (8, 16 or 32)
+template <int LPR>
+__device__ __forceinline__ float dc_group_sum(float v) {
+    if (LPR == 8) return dc_row8_sum(v);
+    v = dc_row16_sum(v);
+    if (LPR == 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+// 8 bf16 (one 16-byte load) dotted with 8 fp32 query values, added to acc
+__device__ __forceinline__ float dc_dot8(const uint4 &w, const float (&q)[8], float acc) {
+    acc = fmaf(dc_bf16_lo(w.x), q[0], acc);
+    acc = fmaf(dc_bf16_hi(w.x), q[1], acc);
+    acc = fmaf(dc_bf16_lo(w.y), q[2], acc);
+    acc = fmaf(dc_bf16_hi(w.y), q[3], acc);
+    acc = fmaf(dc_bf16_lo(w.z), q[4], acc);
+    acc = fmaf(dc_bf16_hi(w.z), q[5], acc);
+    acc = fmaf(dc_bf16_lo(w.w), q[6], acc);
+    acc = fmaf(dc_bf16_hi(w.w), q[7], acc);
+    return acc;
+}

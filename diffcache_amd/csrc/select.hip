@@ -1,0 +1,486 @@
+// Exact top-k selection on fp32 scores.  Replaces the bounded max-heap of
+// search_bruteforce (diffcache_cpu/src/nsw.rs:600-621): the result is the k
+// smallest (ordering key, id) pairs, i.e. the set a size-k heap with the
+// reference's strict "replace on smaller distance" rule ends with (ties go to
+// the lower id), which is also what DualHeap keeps (dualheap.rs:4-87).
+//
+// Three stages, all streaming or tiny:
+//   1. a 4096-bucket histogram of a monotone 12-bit function of the key (filled
+//      by the scoring kernel's epilogue, or by hist_kernel here);
+//   2. filter_kernel: every block finds the bucket tb holding the k-th key,
+//      emits all ids in buckets < tb (certain members) and the (key, id) pairs
+//      of bucket tb (candidates), one atomic per block for each list;
+//   3. finalize_kernel (one block per unit): radix select among the candidates
+//      on the 32-bit key, then on the id among keys equal to the threshold.
+// An optional sort_kernel orders the k ids (best first, or by id).
+#include "dc_common.h"
+
+namespace {
+
+constexpr int kFilterThreads = 256;
+constexpr int kFilterPerThread = 32;
+constexpr int kFilterChunk = kFilterThreads * kFilterPerThread;  // 8192 scores per block
+constexpr int kFinalThreads = 1024;
+constexpr int kRadixBits = 11;
+constexpr int kRadixBins = 1 << kRadixBits;
+constexpr int kSortLds = 4096;
+
+struct UnitMeta {
+    uint32_t tb;        // threshold bucket
+    uint32_t c_less;    // keys in buckets < tb
+    uint32_t win_cnt;   // running count of emitted certain members
+    uint32_t cand_cnt;  // running count of emitted candidates
+};
+
+__global__ void zero_u32_kernel(uint32_t *p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(kFilterThreads) void hist_kernel(
+    const float *__restrict__ scores, int64_t scores_stride, uint32_t *__restrict__ hist,
+    int n_rows, int mode, int blocks_per_unit) {
+    __shared__ uint32_t lhist[DC_HIST_BINS];
+    const int unit = blockIdx.x / blocks_per_unit;
+    const int chunk = blockIdx.x % blocks_per_unit;
+    const int tid = threadIdx.x;
+    for (int i = tid; i < DC_HIST_BINS; i += kFilterThreads) lhist[i] = 0;
+    __syncthreads();
+    const float *su = scores + (int64_t)unit * scores_stride;
+    const int64_t base = (int64_t)chunk * kFilterChunk;
+#pragma unroll 8
+    for (int it = 0; it < kFilterPerThread; ++it) {
+        int64_t i = base + it * kFilterThreads + tid;
+        if (i < n_rows) {
+            uint32_t key, bucket;
+            dc_key_bucket(su[i], mode, key, bucket);
+            atomicAdd(&lhist[bucket], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t *hu = hist + (int64_t)unit * DC_HIST_BINS;
+    for (int i = tid; i < DC_HIST_BINS; i += kFilterThreads) {
+        uint32_t c = lhist[i];
+        if (c) atomicAdd(&hu[i], c);
+    }
+}
+
+// inclusive scan over the lanes of a wave
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        uint32_t t = __shfl_up(v, d, 64);
+        if (lane >= d) v += t;
+    }
+    return v;
+}
+
+// Block-wide exclusive scan for NT threads (NT a multiple of 64, <= 1024).
+// `wtot` is LDS scratch of at least NT/64 + 1 words.  Returns the exclusive
+// prefix; *total receives the block sum.  Contains two barriers.
+template <int NT>
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, uint32_t *total) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int NW = NT / 64;
+    uint32_t incl = wave_incl_scan(v, lane);
+    if (lane == 63) wtot[wave] = incl;
+    __syncthreads();
+    uint32_t off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        uint32_t t = wtot[w];
+        if (w < wave) off += t;
+        tot += t;
+    }
+    __syncthreads();
+    *total = tot;
+    return off + incl - v;
+}
+
+__global__ __launch_bounds__(kFilterThreads) void filter_kernel(
+    const float *__restrict__ scores, int64_t scores_stride, const uint32_t *__restrict__ hist,
+    UnitMeta *__restrict__ meta, uint32_t *__restrict__ idx_out, int64_t idx_stride,
+    uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_idx, int n_rows, int k_eff,
+    int mode, int blocks_per_unit) {
+    __shared__ uint32_t wtot[kFilterThreads / 64 + 1];
+    __shared__ uint32_t s_tb, s_cless, s_wbase, s_cbase;
+    const int unit = blockIdx.x / blocks_per_unit;
+    const int chunk = blockIdx.x % blocks_per_unit;
+    const int tid = threadIdx.x;
+
+    if (tid == 0) {
+        s_tb = DC_HIST_BINS;  // "everything is a certain member" unless a crossing is found
+        s_cless = 0;
+    }
+    // ---- threshold bucket: the bucket holding the k_eff-th smallest key ----
+    uint32_t bins[16];
+    uint32_t sum = 0;
+    {
+        const uint4 *hp = reinterpret_cast<const uint4 *>(hist + (int64_t)unit * DC_HIST_BINS) + tid * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 t = hp[i];
+            bins[4 * i + 0] = t.x;
+            bins[4 * i + 1] = t.y;
+            bins[4 * i + 2] = t.z;
+            bins[4 * i + 3] = t.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += bins[i];
+    }
+    uint32_t total;
+    uint32_t excl = block_excl_scan<kFilterThreads>(sum, wtot, &total);
+    const uint32_t kk = (uint32_t)k_eff;
+    if (excl < kk && kk <= excl + sum) {
+        uint32_t run = excl;
+        bool done = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (!done && run + bins[i] >= kk) {
+                s_tb = tid * 16 + i;
+                s_cless = run;
+                done = true;
+            }
+            run += bins[i];
+        }
+    }
+    __syncthreads();
+    const uint32_t tb = s_tb, c_less = s_cless;
+    if (chunk == 0 && tid == 0) {
+        meta[unit].tb = tb;
+        meta[unit].c_less = c_less;
+    }
+
+    // ---- classify this block's scores ----
+    const float *su = scores + (int64_t)unit * scores_stride;
+    const int64_t base = (int64_t)chunk * kFilterChunk;
+    uint32_t wmask = 0, cmask = 0;
+    uint32_t keys[kFilterPerThread];
+#pragma unroll
+    for (int it = 0; it < kFilterPerThread; ++it) {
+        int64_t i = base + it * kFilterThreads + tid;
+        uint32_t key = 0xffffffffu, bucket = 0xffffffffu;
+        if (i < n_rows) dc_key_bucket(su[i], mode, key, bucket);
+        keys[it] = key;
+        if (i < n_rows) {
+            if (bucket < tb) wmask |= 1u << it;
+            else if (bucket == tb) cmask |= 1u << it;
+        }
+    }
+    const uint32_t nw = __popc(wmask), nc = __popc(cmask);
+    uint32_t tot2;
+    uint32_t ex2 = block_excl_scan<kFilterThreads>(nw | (nc << 16), wtot, &tot2);
+    if (tid == 0) {
+        uint32_t tw = tot2 & 0xffffu, tc = tot2 >> 16;
+        s_wbase = tw ? atomicAdd(&meta[unit].win_cnt, tw) : 0;
+        s_cbase = tc ? atomicAdd(&meta[unit].cand_cnt, tc) : 0;
+    }
+    __syncthreads();
+    uint32_t wpos = s_wbase + (ex2 & 0xffffu);
+    uint32_t cpos = s_cbase + (ex2 >> 16);
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride;
+    uint32_t *ck = cand_key + (int64_t)unit * n_rows;
+    uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
+#pragma unroll
+    for (int it = 0; it < kFilterPerThread; ++it) {
+        uint32_t i = (uint32_t)(base + it * kFilterThreads + tid);
+        if (wmask & (1u << it)) {
+            if (wpos < kk) io[wpos] = i;
+            ++wpos;
+        } else if (cmask & (1u << it)) {
+            if (cpos < (uint32_t)n_rows) {
+                ck[cpos] = keys[it];
+                ci[cpos] = i;
+            }
+            ++cpos;
+        }
+    }
+}
+
+// Among `n` values v(i), find the rem-th smallest (1-based) by radix passes over
+// bits [hb, 0].  get(i, &value) returns false for items outside the subset.
+// Returns the threshold value; *rem_out = how many items equal to it are needed
+// (rank of the threshold inside its tie group), *n_eq = size of the tie group.
+template <typename Get>
+__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int hb, uint32_t common,
+                                       uint32_t *lh, uint32_t *wtot, uint32_t *sres,
+                                       uint32_t *rem_out, uint32_t *n_eq) {
+    const int tid = threadIdx.x;
+    uint32_t prefix = common;  // bits above hb, shared by every item
+    int top = hb + 1;          // bits [top-1, 0] still undecided
+    uint32_t eq = n;
+    while (top > 0) {
+        const int width = top < kRadixBits ? top : kRadixBits;
+        const int shift = top - width;
+        for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
+        __syncthreads();
+        const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
+        for (uint32_t i = tid; i < n; i += kFinalThreads) {
+            uint32_t v;
+            if (get(i, &v) && ((v & himask) == (prefix & himask)))
+                atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
+        }
+        __syncthreads();
+        // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
+        const uint32_t h0 = lh[2 * tid], h1 = lh[2 * tid + 1];
+        uint32_t total;
+        const uint32_t excl = block_excl_scan<kFinalThreads>(h0 + h1, wtot, &total);
+        if (excl < rem && rem <= excl + h0 + h1) {
+            if (excl + h0 >= rem) {
+                sres[0] = 2 * tid;
+                sres[1] = excl;
+                sres[2] = h0;
+            } else {
+                sres[0] = 2 * tid + 1;
+                sres[1] = excl + h0;
+                sres[2] = h1;
+            }
+        }
+        __syncthreads();
+        prefix |= sres[0] << shift;
+        rem -= sres[1];
+        eq = sres[2];
+        top = shift;
+        __syncthreads();
+    }
+    *rem_out = rem;
+    *n_eq = eq;
+    return prefix;
+}
+
+__global__ __launch_bounds__(kFinalThreads) void finalize_kernel(
+    const UnitMeta *__restrict__ meta, const uint32_t *__restrict__ cand_key,
+    const uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out, int64_t idx_stride,
+    int n_rows, int k_eff) {
+    __shared__ uint32_t lh[kRadixBins];
+    __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
+    __shared__ uint32_t sres[4];
+    __shared__ uint32_t s_diff, s_slot;
+    const int unit = blockIdx.x;
+    const int tid = threadIdx.x;
+    const uint32_t c_less = meta[unit].c_less;
+    uint32_t n_c = meta[unit].cand_cnt;
+    if (n_c > (uint32_t)n_rows) n_c = n_rows;
+    if (c_less >= (uint32_t)k_eff) return;
+    uint32_t need = (uint32_t)k_eff - c_less;
+    if (need > n_c) need = n_c;
+    const uint32_t *ck = cand_key + (int64_t)unit * n_rows;
+    const uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride + c_less;
+
+    if (need == n_c) {  // the whole threshold bucket is selected
+        for (uint32_t i = tid; i < n_c; i += kFinalThreads) io[i] = ci[i];
+        return;
+    }
+
+    // bits in which the candidate keys differ
+    if (tid == 0) {
+        s_diff = 0;
+        s_slot = 0;
+    }
+    __syncthreads();
+    const uint32_t k0 = ck[0];
+    uint32_t diff = 0;
+    for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
+    if (diff) atomicOr(&s_diff, diff);
+    __syncthreads();
+    diff = s_diff;
+    const int hb = diff ? 31 - __clz(diff) : -1;
+    const uint32_t common = (hb >= 31) ? 0u : (k0 & (0xffffffffu << (hb + 1)));
+
+    uint32_t need_eq, n_eq;
+    auto get_key = [&](uint32_t i, uint32_t *v) {
+        *v = ck[i];
+        return true;
+    };
+    const uint32_t t_key =
+        block_radix_select(get_key, n_c, need, hb, common, lh, wtot, sres, &need_eq, &n_eq);
+
+    uint32_t t_idx = 0xffffffffu;
+    if (need_eq < n_eq) {  // only the lowest ids of the tie group fit
+        const uint32_t span = (uint32_t)(n_rows - 1) | 1u;
+        const int hbi = 31 - __clz(span);
+        auto get_idx = [&](uint32_t i, uint32_t *v) {
+            *v = ci[i];
+            return ck[i] == t_key;
+        };
+        uint32_t r2, e2;
+        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi, 0u, lh, wtot, sres, &r2, &e2);
+    }
+
+    for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
+        const uint32_t key = ck[i], id = ci[i];
+        if (key < t_key || (key == t_key && id <= t_idx)) {
+            uint32_t slot = atomicAdd(&s_slot, 1u);
+            if (slot < need) io[slot] = id;
+        }
+    }
+}
+
+// Bitonic sort of each unit's k ids by (key, id) or by id.
+template <bool IN_LDS>
+__global__ __launch_bounds__(kFinalThreads) void sort_kernel(
+    const float *__restrict__ scores, int64_t scores_stride, uint32_t *__restrict__ idx_out,
+    int64_t idx_stride, unsigned long long *__restrict__ scratch, int k_eff, int pow2, int mode,
+    int order) {
+    __shared__ unsigned long long lbuf[IN_LDS ? kSortLds : 1];
+    const int unit = blockIdx.x;
+    const int tid = threadIdx.x;
+    unsigned long long *buf = IN_LDS ? lbuf : scratch + (int64_t)unit * pow2;
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride;
+    const float *su = scores + (int64_t)unit * scores_stride;
+    for (int i = tid; i < pow2; i += kFinalThreads) {
+        unsigned long long v = ~0ull;
+        if (i < k_eff) {
+            uint32_t id = io[i];
+            if (order == DC_ORDER_BEST) {
+                uint32_t key, bucket;
+                dc_key_bucket(su[id], mode, key, bucket);
+                v = ((unsigned long long)key << 32) | id;
+            } else {
+                v = id;
+            }
+        }
+        buf[i] = v;
+    }
+    __syncthreads();
+    for (int size = 2; size <= pow2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int t = tid; t < (pow2 >> 1); t += kFinalThreads) {
+                const int i = ((t / stride) * 2 * stride) + (t % stride);
+                const int j = i + stride;
+                const bool asc = (i & size) == 0;
+                unsigned long long a = buf[i], b = buf[j];
+                if ((a > b) == asc) {
+                    buf[i] = b;
+                    buf[j] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for (int i = tid; i < k_eff; i += kFinalThreads) io[i] = (uint32_t)(buf[i] & 0xffffffffull);
+}
+
+__global__ void compose_idx_kernel(const uint32_t *__restrict__ outer, int64_t outer_stride,
+                                   const uint32_t *__restrict__ inner, int64_t inner_stride,
+                                   uint32_t *__restrict__ out, int64_t out_stride, int n_inner,
+                                   int64_t total) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    int64_t u = t / n_inner, j = t % n_inner;
+    out[u * out_stride + j] = outer[u * outer_stride + inner[u * inner_stride + j]];
+}
+
+struct SelectWs {
+    uint32_t *hist;
+    UnitMeta *meta;
+    uint32_t *cand_key, *cand_idx;
+    unsigned long long *sort_scratch;
+    size_t bytes;
+};
+
+int next_pow2(int x) {
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+SelectWs carve(void *base, int n_units, int n_rows, int k) {
+    SelectWs w;
+    size_t off = 0;
+    char *p = (char *)base;
+    w.hist = (uint32_t *)(p + off);
+    off += dc_align_up((size_t)n_units * DC_HIST_BINS * 4, 256);
+    w.meta = (UnitMeta *)(p + off);
+    off += dc_align_up((size_t)n_units * sizeof(UnitMeta), 256);
+    w.cand_key = (uint32_t *)(p + off);
+    off += dc_align_up((size_t)n_units * (size_t)n_rows * 4, 256);
+    w.cand_idx = (uint32_t *)(p + off);
+    off += dc_align_up((size_t)n_units * (size_t)n_rows * 4, 256);
+    w.sort_scratch = (unsigned long long *)(p + off);
+    int keff = k < n_rows ? k : n_rows;
+    if (keff > kSortLds) off += dc_align_up((size_t)n_units * next_pow2(keff) * 8, 256);
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" size_t dc_topk_workspace_bytes(int n_units, int n_rows, int k) {
+    if (n_units <= 0 || n_rows <= 0 || k <= 0) return 256;
+    return carve(nullptr, n_units, n_rows, k).bytes;
+}
+
+extern "C" int dc_topk_select(const float *scores, int64_t scores_unit_stride, uint32_t *idx_out,
+                              int64_t idx_unit_stride, int n_units, int n_rows, int k, int mode,
+                              int order, const uint32_t *hist, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(scores && idx_out, "dc_topk_select: null pointer");
+    DC_REQUIRE(n_units >= 0 && n_rows >= 0 && k >= 0, "dc_topk_select: bad sizes");
+    DC_REQUIRE(mode == DC_MODE_IP || mode == DC_MODE_REF_DIST, "dc_topk_select: bad mode %d", mode);
+    DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "dc_topk_select: bad order %d", order);
+    const int k_eff = k < n_rows ? k : n_rows;
+    if (n_units == 0 || k_eff == 0) return DC_OK;
+    DC_REQUIRE(scores_unit_stride >= n_rows, "dc_topk_select: scores_unit_stride < n_rows");
+    DC_REQUIRE(idx_unit_stride >= k_eff, "dc_topk_select: idx_unit_stride < min(k, n_rows)");
+    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
+               "dc_topk_select: workspace must be non-null and 256-byte aligned");
+    DC_REQUIRE(!hist || dc_aligned16(hist), "dc_topk_select: hist must be 16-byte aligned");
+    SelectWs w = carve(workspace, n_units, n_rows, k);
+    if (workspace_bytes < w.bytes) {
+        dc_set_error("dc_topk_select: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
+        return DC_ENOMEM;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t bpu = ((int64_t)n_rows + kFilterChunk - 1) / kFilterChunk;
+    DC_REQUIRE((int64_t)n_units * bpu < (1ll << 31), "dc_topk_select: grid too large");
+
+    // clear the running counters (and the histogram if it is computed here)
+    {
+        uint32_t *z = hist ? (uint32_t *)w.meta : w.hist;
+        int64_t n = ((char *)w.cand_key - (char *)z) / 4;
+        hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, z, n);
+        DC_CHECK_LAUNCH("dc_topk_select(zero)");
+    }
+    if (!hist) {
+        hipLaunchKernelGGL(hist_kernel, dim3((unsigned)(n_units * bpu)), dim3(kFilterThreads), 0, st,
+                           scores, scores_unit_stride, w.hist, n_rows, mode, (int)bpu);
+        DC_CHECK_LAUNCH("dc_topk_select(hist)");
+        hist = w.hist;
+    }
+    hipLaunchKernelGGL(filter_kernel, dim3((unsigned)(n_units * bpu)), dim3(kFilterThreads), 0, st,
+                       scores, scores_unit_stride, hist, w.meta, idx_out, idx_unit_stride,
+                       w.cand_key, w.cand_idx, n_rows, k_eff, mode, (int)bpu);
+    DC_CHECK_LAUNCH("dc_topk_select(filter)");
+    hipLaunchKernelGGL(finalize_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.meta,
+                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, n_rows, k_eff);
+    DC_CHECK_LAUNCH("dc_topk_select(finalize)");
+    if (order != DC_ORDER_ANY) {
+        const int p2 = next_pow2(k_eff);
+        if (p2 <= kSortLds)
+            hipLaunchKernelGGL(sort_kernel<true>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
+                               scores_unit_stride, idx_out, idx_unit_stride,
+                               (unsigned long long *)nullptr, k_eff, p2, mode, order);
+        else
+            hipLaunchKernelGGL(sort_kernel<false>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
+                               scores_unit_stride, idx_out, idx_unit_stride, w.sort_scratch, k_eff,
+                               p2, mode, order);
+        DC_CHECK_LAUNCH("dc_topk_select(sort)");
+    }
+    return DC_OK;
+}
+
+extern "C" int dc_compose_idx(const uint32_t *outer, int64_t outer_unit_stride,
+                              const uint32_t *inner, int64_t inner_unit_stride, uint32_t *out,
+                              int64_t out_unit_stride, int n_units, int n_inner, void *stream) {
+    DC_REQUIRE(outer && inner && out, "dc_compose_idx: null pointer");
+    DC_REQUIRE(n_units >= 0 && n_inner >= 0, "dc_compose_idx: bad sizes");
+    int64_t total = (int64_t)n_units * n_inner;
+    if (total == 0) return DC_OK;
+    hipLaunchKernelGGL(compose_idx_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, outer, outer_unit_stride, inner, inner_unit_stride, out,
+                       out_unit_stride, n_inner, total);
+    DC_CHECK_LAUNCH("dc_compose_idx");
+    return DC_OK;
+}

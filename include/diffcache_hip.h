@@ -1,0 +1,223 @@
+/*
+ * diffcache_hip.h -- C ABI of libdiffcache_hip.so: the decode-time retrieval
+ * path of DiffCache on one MI355X (gfx950), K/V resident in HBM as bf16.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes and element strides (no torch types);
+ *   - enqueues its kernels on `stream` (a hipStream_t passed as void*) and
+ *     returns without synchronising; nothing is allocated or freed, so the
+ *     calls can sit between the two captured graph halves of a decode layer;
+ *   - returns 0 on success or a negative DC_E* code, with a message kept for
+ *     dc_last_error() (the reference panics instead: lib.rs:294,332,353,376,579).
+ *
+ * bf16 crosses the boundary as raw 16-bit words, as in the reference
+ * (diffcache_cpu/src/lib.rs:529-544).  A "unit" is one (batch, kv-head) pair:
+ * the reference keeps one independent index per unit (lib.rs:189-197,296-313).
+ * Row r of unit (b, h) of a K or V store starts at element
+ *   b * batch_stride + h * head_stride + r * row_stride
+ * with head_dim contiguous bf16 values; all strides are in elements, must be
+ * multiples of 8 and the base pointers 16-byte aligned.
+ *
+ * Paths in comments are relative to the reference checkout.
+ */
+#ifndef DIFFCACHE_HIP_H
+#define DIFFCACHE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DC_VERSION 1
+
+/* ordering-key modes */
+#define DC_MODE_IP 0       /* highest inner product first, ties -> lower index */
+#define DC_MODE_REF_DIST 1 /* order by f32(65536 - ip) as nsw.rs:138 does, ties -> lower index */
+
+/* order of the selected ids */
+#define DC_ORDER_ANY 0    /* unspecified (fastest) */
+#define DC_ORDER_BEST 1   /* ascending (key, id): the order nsw.rs:621-629 writes rows in */
+#define DC_ORDER_INDEX 2  /* ascending id */
+
+/* error codes */
+#define DC_OK 0
+#define DC_EINVAL (-22)
+#define DC_ENOMEM (-12)   /* workspace too small */
+#define DC_ELAUNCH (-5)   /* hipLaunchKernel failed */
+
+#define DC_HIST_BINS 4096 /* coarse histogram bins per unit used by the select */
+
+/* Library version (DC_VERSION).  Replaces nothing; added for binding checks. */
+int dc_version(void);
+
+/* Message of the last failing call on this thread ("" if none).
+ * Replaces the Rust panic text surfaced as PanicException (lib.rs:294-579). */
+const char *dc_last_error(void);
+
+/*
+ * GQA-group mean query, rounded to bf16.
+ * q (n_units, group, hd) bf16 -> q_mean (n_units, hd) bf16: fp32 sum over the
+ * group, one division, round to nearest even.
+ * Replaces src/diffcache/kvcache/diffcache.py:191-194 (view(b,Hkv,G,hd).mean(2)).
+ */
+int dc_group_mean_bf16(const void *q, void *q_mean, int n_units, int group, int hd, void *stream);
+
+/*
+ * Inner-product scores of one query per unit against n_rows key rows.
+ *   k       first row to score of unit (0,0)
+ *   q       (n_b*n_h, q_group, hd) bf16.  q_group == 1: the query itself;
+ *           q_group > 1: the GQA group, averaged as dc_group_mean_bf16 does
+ *   scores  out, fp32, unit u at scores + u*scores_unit_stride, n_rows each
+ *   hist    NULL, or (n_b*n_h, DC_HIST_BINS) uint32 zeroed by the caller: receives
+ *           the coarse histogram of the ordering keys that dc_topk_select needs
+ * Products of bf16 values are exact in fp32; accumulation is fp32.
+ * Replaces Index::distance(QKDist) over the scan of search_bruteforce
+ * (diffcache_cpu/src/nsw.rs:129-139,601-607; simsimd dot, lib.rs:65-69).
+ */
+int dc_score_bf16(const void *k, const void *q, float *scores, uint32_t *hist, int n_b, int n_h,
+                  int n_rows, int hd, int64_t k_batch_stride, int64_t k_head_stride,
+                  int64_t k_row_stride, int64_t scores_unit_stride, int q_group, int mode,
+                  void *stream);
+
+/* Bytes of workspace dc_topk_select needs for these sizes. */
+size_t dc_topk_workspace_bytes(int n_units, int n_rows, int k);
+
+/*
+ * Exact top-k of each unit's scores: the min(k, n_rows) smallest
+ * (ordering key, id) pairs, where the key is given by `mode`.
+ *   idx_out (n_units, idx_unit_stride) uint32: ids in [0, n_rows); the first
+ *           min(k, n_rows) entries of each unit are written, in `order`
+ *   hist    NULL (computed here) or the histogram dc_score_bf16 filled
+ *   workspace  dc_topk_workspace_bytes(...) bytes, 256-byte aligned
+ * Replaces the bounded max-heap scan and ascending collect of
+ * search_bruteforce (diffcache_cpu/src/nsw.rs:600-621), the u64 key packing
+ * (nsw.rs:74-91) and the kept-set semantic of DualHeap (dualheap.rs:4-87).
+ */
+int dc_topk_select(const float *scores, int64_t scores_unit_stride, uint32_t *idx_out,
+                   int64_t idx_unit_stride, int n_units, int n_rows, int k, int mode, int order,
+                   const uint32_t *hist, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Copy selected K and V rows into dense output buffers.
+ * For unit (b, h) and j < n_idx:
+ *   out_k[b, h, j, :] = k[b, h, row_offset + idx[u, j], :]   (same for v)
+ * idx unit u = b*n_h + h at idx + u*idx_unit_stride.
+ * Replaces the row gather of search_bruteforce (nsw.rs:621-629) together with
+ * the pinned-buffer hop and H2D copies of
+ * src/diffcache/kvcache/diffcache.py:196-209.
+ */
+int dc_gather_rows_bf16(const void *k, const void *v, const uint32_t *idx, void *out_k, void *out_v,
+                        int n_b, int n_h, int n_idx, int64_t idx_unit_stride, int hd,
+                        int64_t row_offset, int64_t src_batch_stride, int64_t src_head_stride,
+                        int64_t src_row_stride, int64_t dst_batch_stride, int64_t dst_head_stride,
+                        int64_t dst_row_stride, void *stream);
+
+/* Bytes of workspace dc_gather_attn_bf16 needs. */
+size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attended);
+
+/*
+ * Decode attention over a gathered set of rows, for the `group` query heads
+ * that share each kv-head.  For unit (b, h) the attended rows are
+ *   region_lo + idx[u, j]        j < n_idx     (the retrieved rows)
+ *   [0, n_sink)                                 (prefix, always kept)
+ *   [recent_lo, recent_lo + n_recent)           (suffix, always kept)
+ *   new_k/new_v[u, :]            if not NULL    (the current token)
+ * q, out: (n_b, n_h*group, hd) bf16, query head h*group + g belongs to kv-head h.
+ * out = softmax(q . K^T * scale) . V, fp32 softmax and accumulation, bf16 out;
+ * lse (n_b, n_h*group) fp32 log-sum-exp of the scaled logits, or NULL.
+ * Replaces flash_attn_with_kvcache over the assembled buffer
+ * (src/diffcache/base.py:134-142) and the buffer assembly it reads
+ * (src/diffcache/kvcache/diffcache.py:48-66,186-209).
+ */
+int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
+                        const void *new_k, const void *new_v, void *out, float *lse, int n_b,
+                        int n_h, int group, int hd, int n_idx, int64_t idx_unit_stride,
+                        int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
+                        int64_t k_batch_stride, int64_t k_head_stride, int64_t k_row_stride,
+                        int64_t v_batch_stride, int64_t v_head_stride, int64_t v_row_stride,
+                        float scale, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Append one token: k_store[b, h, pos, :] = new_k[b, h, :] (same for v).
+ * new_k/new_v (n_b, n_h, hd) contiguous.
+ * Replaces DataLayer::insert / Index::insert's row write
+ * (diffcache_cpu/src/lib.rs:352-369, nsw.rs:551-557); no graph is built.
+ */
+int dc_append_kv_bf16(void *k_store, void *v_store, const void *new_k, const void *new_v, int n_b,
+                      int n_h, int hd, int64_t pos, int64_t batch_stride, int64_t head_stride,
+                      int64_t row_stride, void *stream);
+
+/*
+ * Prefill ingest: src (n_b, seq, n_h, hd) -> store[b, h, dst_pos + s, :].
+ * Replaces the permute(0,2,1,3).contiguous() + host copy + Index::prefill memcpy
+ * (src/diffcache/kvcache/diffcache.py:142-147, diffcache_cpu/src/nsw.rs:503-508).
+ */
+int dc_ingest_kv_bf16(void *store, const void *src, int n_b, int seq, int n_h, int hd,
+                      int64_t dst_pos, int64_t batch_stride, int64_t head_stride,
+                      int64_t row_stride, void *stream);
+
+/*
+ * One decode layer of the path: score -> select -> attend, enqueued back to back.
+ * All pointers are device pointers; see the single-step calls for the meaning
+ * of each field.  n_ctx rows are valid per unit; the retrieval region is
+ * [n_sink, recent_lo); ids written to idx_out are relative to n_sink (the
+ * reference's node ids are relative to the region too: diffcache.py:175-181).
+ * Replaces the call sequence of BaseModel.layer_decode
+ * (src/diffcache/base.py:150-155) between the two captured graph halves.
+ */
+typedef struct dc_layer_args {
+    const void *q;        /* (n_b, n_h*group, hd) bf16 */
+    const void *k;        /* K store */
+    const void *v;        /* V store */
+    const void *new_k;    /* (n_b, n_h, hd) bf16 or NULL */
+    const void *new_v;
+    void *out;            /* (n_b, n_h*group, hd) bf16 */
+    float *lse;           /* (n_b, n_h*group) or NULL */
+    float *scores;        /* (n_units, scores_unit_stride) fp32 scratch/output */
+    uint32_t *idx_out;    /* (n_units, idx_unit_stride) */
+    void *workspace;      /* dc_layer_workspace_bytes(...) bytes, 256-byte aligned */
+    size_t workspace_bytes;
+    int64_t kv_batch_stride, kv_head_stride, kv_row_stride; /* same for K and V */
+    int64_t scores_unit_stride, idx_unit_stride;
+    int64_t recent_lo;    /* first row of the always-kept suffix */
+    int n_b, n_h, group, hd;
+    int n_sink, n_recent; /* rows [0,n_sink) and [recent_lo, recent_lo+n_recent) always kept */
+    int budget;           /* k */
+    int mode, order;
+    float scale;          /* softmax scale, 1/sqrt(hd) in the reference */
+} dc_layer_args;
+
+size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,
+                                int n_rows_attended);
+int dc_decode_layer(const dc_layer_args *args, void *stream);
+
+/*
+ * PQ asymmetric-distance baseline.  The reference's PQ baseline directory
+ * (evaluation/impl/pqcache) is empty, so these replace no reference code; the
+ * shapes follow the benchmark configuration (M subspaces x 256 centroids).
+ *   dc_pq_build_lut: lut[u, m, c] = q[u, m*ds:(m+1)*ds] . books[h(u), m, c, :]
+ *     q (n_b*n_h, hd) bf16, books (n_h, M, 256, ds) fp32, lut (n_b*n_h, M, 256) fp32
+ *   dc_pq_adc_scan: scores[u, i] = sum_m lut[u, m, codes[u, i, m]]
+ *     codes (n_units, n_rows, M) uint8, fp32 adds in ascending m;
+ *     hist as in dc_score_bf16 (keys in DC_MODE_IP order), or NULL
+ *   dc_score_gathered_bf16: scores[u, j] = q[u] . k[row_offset + idx[u, j]]  (exact rerank)
+ *   dc_compose_idx: out[u, j] = outer[u, inner[u, j]]
+ */
+int dc_pq_build_lut(const void *q, const float *books, float *lut, int n_b, int n_h, int hd, int m,
+                    void *stream);
+int dc_pq_adc_scan(const uint8_t *codes, const float *lut, float *scores, uint32_t *hist,
+                   int n_units, int n_rows, int m, int64_t scores_unit_stride, void *stream);
+int dc_score_gathered_bf16(const void *k, const void *q, const uint32_t *idx, float *scores,
+                           int n_b, int n_h, int n_idx, int64_t idx_unit_stride, int hd,
+                           int64_t row_offset, int64_t k_batch_stride, int64_t k_head_stride,
+                           int64_t k_row_stride, int64_t scores_unit_stride, void *stream);
+int dc_compose_idx(const uint32_t *outer, int64_t outer_unit_stride, const uint32_t *inner,
+                   int64_t inner_unit_stride, uint32_t *out, int64_t out_unit_stride, int n_units,
+                   int n_inner, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DIFFCACHE_HIP_H */

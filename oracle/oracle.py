@@ -450,3 +450,18 @@ def pq_search(q_u16: np.ndarray, k_u16: np.ndarray, codes: np.ndarray, lut_f32: 
     packed = (key32(exact, MODE_IP).astype(np.uint64) << np.uint64(32)) | cand.astype(np.uint64)
     packed = np.sort(packed)[:min(k, len(cand))]
     return cand, (packed & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+
+
+# --------------------------------------------------------------------------
+# Checking aid for the HIP select's internal histogram (no reference
+# counterpart): the 12-bit monotone bucket of an ordering key.
+# --------------------------------------------------------------------------
+
+
+def coarse_bucket(scores: np.ndarray, mode: int) -> np.ndarray:
+    s = np.asarray(scores, dtype=np.float32)
+    if mode == MODE_REF_DIST:
+        d = ref_dist(s)
+        s = (np.float32(65536.0) - d).astype(np.float32)
+    s = (s + np.float32(0.0)).astype(np.float32)
+    return (_f2ord((-s).astype(np.float32)) >> np.uint32(20)).astype(np.uint32)
