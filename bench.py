@@ -1,0 +1,253 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode-time retrieval path on one MI355X.
+
+Workload (default): BASELINE.json configs[2] -- a full 32-layer Llama-3-8B-shaped
+decode step, batch 8, context 131072 per sequence, 32 query / 8 kv heads,
+head_dim 128, bf16 K/V resident in HBM (~137 GB), top-k 2048 plus 4 sink tokens
+and a 64-token recent window.  One "step" = for every layer: score the whole
+retrieval region with the GQA-mean query, select the exact top-k, run the
+gathered attention (including the current token's k/v).  Inputs are synthetic
+and already in HBM when the timed region starts.
+
+Prints ONE JSON line (see README / DESIGN for the fields).  `value` is the
+latency of one whole decode step in microseconds (lower is better).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+CONFIGS = {
+    # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
+    "c3": dict(layers=32, batch=8, hq=32, hkv=8, hd=128, ctx=131072, budget=2048, sink=4, recent=64,
+               desc="config3: 32-layer Llama-3-8B-shaped decode step, batch 8, ctx 131072, "
+                    "32q/8kv heads, hd 128, bf16 K/V in HBM, top-k 2048 + 4 sinks + 64 recent"),
+    "c2": dict(layers=1, batch=1, hq=32, hkv=8, hd=128, ctx=32768, budget=1024, sink=4, recent=64,
+               desc="config2: one Llama-3-8B-shaped decode layer, batch 1, ctx 32768, "
+                    "top-k 1024 + 4 sinks + 64 recent"),
+    "c5": dict(layers=32, batch=1, hq=32, hkv=8, hd=128, ctx=1048576, budget=4096, sink=4, recent=64,
+               desc="config5: 32 layers, batch 1, ctx 1048576, top-k 4096 + 4 sinks + 64 recent"),
+}
+
+
+def algorithmic_bytes_per_unit(n_region: int, attended: int, group: int, hd: int) -> int:
+    """K streamed once + gathered K and V rows + q in / out (bf16)."""
+    return n_region * hd * 2 + 2 * attended * hd * 2 + group * hd * 2 * 2
+
+
+def make_layer(torch, cfg, layer: int, cfg_id: int, dev):
+    """Synthetic K, V, q, new k/v of one layer, generated on the device."""
+    g = torch.Generator(device=dev).manual_seed(1000 * cfg_id + layer)
+    b, hkv, hq, hd, n = cfg["batch"], cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"]
+    k = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    v = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    k.normal_(generator=g)
+    v.normal_(generator=g)
+    # per-channel log-normal scale (sigma 1), one vector per kv head: outlier channels
+    scale = torch.exp(torch.randn((1, hkv, 1, hd), generator=g, device=dev)).to(torch.bfloat16)
+    k.mul_(scale)
+    # queries: 0.7 * mean of a random 32-key cluster + 0.3 * N(0,1), per query head
+    grp = hq // hkv
+    pick = torch.randint(0, n, (b, hq, 32), generator=g, device=dev)
+    bi = torch.arange(b, device=dev).view(b, 1, 1).expand(b, hq, 32)
+    hi = (torch.arange(hq, device=dev) // grp).view(1, hq, 1).expand(b, hq, 32)
+    centre = k[bi, hi, pick].float().mean(dim=2)
+    q = (0.7 * centre + 0.3 * torch.randn((b, hq, hd), generator=g, device=dev)).to(torch.bfloat16)
+    new_k = torch.randn((b, hkv, hd), generator=g, device=dev).to(torch.bfloat16)
+    new_v = torch.randn((b, hkv, hd), generator=g, device=dev).to(torch.bfloat16)
+    return k, v, q.contiguous(), new_k, new_v
+
+
+def cpu_baseline(torch, cfg, layers_data, target_s: float = 12.0):
+    """The C restatement of the reference's exact-scan path, timed on this box's
+    host cores on a bounded sample: layer 0, batch element 0 (hkv units), one
+    thread per unit like rayon's fan-out, repeated until ~target_s of work."""
+    import numpy as np
+    from oracle import cpu_ref
+    k, v, q, nk, nv = layers_data[0]
+    hkv, hq, hd, n = cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"]
+    grp = hq // hkv
+
+    def host(t):
+        return t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+    k0, v0 = host(k[0]), host(v[0])                       # (hkv, n, hd)
+    q0 = host(q[0]).reshape(hkv, grp, hd)
+    nk0, nv0 = host(nk[0]), host(nv[0])
+    cores = os.cpu_count() or 1
+    # the GPU box gives one GPU's share of the host: 16 cores
+    threads = min(hkv, cores, 16)
+    cpu_ref.lib()
+    reps, total = 0, 0.0
+    t_first = None
+    while total < target_s and reps < 64:
+        t0 = time.perf_counter()
+        cpu_ref.decode_layer(q0, k0, v0, cfg["budget"], cfg["sink"], cfg["recent"], n_ctx=n,
+                             new_k_u16=nk0, new_v_u16=nv0, n_threads=threads, want_ids=False)
+        dt = time.perf_counter() - t0
+        t_first = dt if t_first is None else t_first
+        total += dt
+        reps += 1
+    per_sample = total / reps
+    units_total = cfg["layers"] * cfg["batch"] * hkv
+    step_us = per_sample * (units_total / hkv) * 1e6
+    return {
+        "value": step_us, "unit": "us", "cores": threads, "kind": "port",
+        "sample": (f"oracle/cpu_ref.c decode_layer on layer 0, batch element 0 ({hkv} units x {n} rows), "
+                   f"{threads} threads, mean of {reps} runs = {per_sample * 1e3:.1f} ms; scaled x"
+                   f"{units_total // hkv} to the full step ({cfg['layers']} layers x batch {cfg['batch']}); "
+                   f"host reports {cores} cpus"),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
+    ap.add_argument("--mode", default="ref_dist", choices=["ref_dist", "ip"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--fused", action="store_true",
+                    help="time dc_decode_layer (one call per layer) instead of the split calls")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
+              "use --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from diffcache_amd import _hip as hip
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = CONFIGS[args.config]
+    cfg_id = {"c2": 2, "c3": 3, "c5": 5}[args.config]
+    mode = hip.MODE_REF_DIST if args.mode == "ref_dist" else hip.MODE_IP
+    L, b, hq, hkv, hd, n = cfg["layers"], cfg["batch"], cfg["hq"], cfg["hkv"], cfg["hd"], cfg["ctx"]
+    grp = hq // hkv
+    n_units = b * hkv
+    sink, recent, budget = cfg["sink"], cfg["recent"], cfg["budget"]
+    lo, hi = sink, n - recent
+    region = hi - lo
+    k_eff = min(budget, region)
+    attended = k_eff + sink + recent + 1
+
+    t_gen = time.perf_counter()
+    layers = [make_layer(torch, cfg, l, cfg_id, dev) for l in range(L)]
+    torch.cuda.synchronize()
+    t_gen = time.perf_counter() - t_gen
+
+    scores = torch.empty((n_units, region), dtype=torch.float32, device=dev)
+    idx = torch.empty((n_units, budget), dtype=torch.int32, device=dev)
+    out = torch.empty((b, hq, hd), dtype=torch.bfloat16, device=dev)
+    hist = hip.new_hist(n_units, dev)
+    ws_topk = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(n_units, region, budget), dev)
+    ws_attn = hip.alloc_workspace(hip.lib.dc_attn_workspace_bytes(n_units, grp, hd, attended), dev)
+    ws_layer = hip.alloc_workspace(hip.layer_workspace_bytes(n_units, region, budget, grp, hd, attended), dev)
+
+    def new_events(count):
+        return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+
+    def step(ev=None):
+        """One decode step: every layer, in order, on the current stream."""
+        for l in range(L):
+            k, v, q, nk, nv = layers[l]
+            if args.fused:
+                hip.decode_layer(q, k, v, sink, hi, recent, budget, scores, idx, out, ws_layer, nk, nv,
+                                 mode=mode, order=hip.ORDER_ANY)
+                continue
+            hist.zero_()
+            if ev is not None:
+                ev[4 * l + 0].record()
+            hip.score(k, q, lo, region, mode, q_group=grp, scores=scores, hist=hist)
+            if ev is not None:
+                ev[4 * l + 1].record()
+            hip.topk_select(scores, budget, mode, hip.ORDER_ANY, hist=hist, idx_out=idx,
+                            workspace=ws_topk)
+            if ev is not None:
+                ev[4 * l + 2].record()
+            hip.gather_attn(q, k, v, idx, k_eff, lo, sink, hi, recent, nk, nv, out=out,
+                            workspace=ws_attn)
+            if ev is not None:
+                ev[4 * l + 3].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [new_events(4 * L) for _ in range(args.steps)] if not args.fused else None
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        step(None if events is None else events[s])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-kernel durations from the events of the timed region
+    stage_us = None
+    score_ms = None
+    if events is not None:
+        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in events for l in range(L)]
+        se = [e[4 * l + 1].elapsed_time(e[4 * l + 2]) for e in events for l in range(L)]
+        at = [e[4 * l + 2].elapsed_time(e[4 * l + 3]) for e in events for l in range(L)]
+        score_ms = sum(sc) / len(sc)
+        stage_us = {"score": score_ms * 1e3, "select": sum(se) / len(se) * 1e3,
+                    "attn": sum(at) / len(at) * 1e3}
+
+    unit_bytes = algorithmic_bytes_per_unit(region, k_eff + sink + recent, grp, hd)
+    step_bytes = unit_bytes * n_units * L
+    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    score_bytes = n_units * region * hd * 2          # K rows streamed by one score launch
+    roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
+                "traffic": None, "kernel": "score_kernel<128>",
+                "algorithmic_bytes_per_launch": score_bytes}
+    if score_ms is not None:
+        ach = score_bytes / (score_ms * 1e-3) / 1e9
+        roofline.update(achieved=ach, frac=ach / HBM_PEAK_GBPS, avg_launch_us=score_ms * 1e3)
+
+    result = {
+        "metric": "decode_step_retrieval_sparse_attn_latency_us",
+        "value": ms_per_step * 1e3,
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": cfg["desc"], "key_mode": args.mode,
+                   "call_path": "dc_decode_layer" if args.fused else "dc_score/dc_topk_select/dc_gather_attn"},
+        "step_hbm_gbps": step_gbps,
+        "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
+        "step_algorithmic_bytes": step_bytes,
+        "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
+        "stage_us_per_layer": stage_us,
+        "roofline": roofline,
+        "setup_s": t_gen,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, cfg, layers)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
