@@ -120,6 +120,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--fused", action="store_true",
                     help="time dc_decode_layer (one call per layer) instead of the split calls")
+    ap.add_argument("--dense", action="store_true",
+                    help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
+                         "streaming score + select")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
@@ -158,6 +161,7 @@ def main() -> int:
     ws_topk = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(n_units, region, budget), dev)
     ws_attn = hip.alloc_workspace(hip.lib.dc_attn_workspace_bytes(n_units, grp, hd, attended), dev)
     ws_layer = hip.alloc_workspace(hip.layer_workspace_bytes(n_units, region, budget, grp, hd, attended), dev)
+    ws_sel = hip.alloc_workspace(hip.score_select_workspace_bytes(n_units, region, budget), dev)
 
     def new_events(count):
         return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
@@ -167,17 +171,26 @@ def main() -> int:
         for l in range(L):
             k, v, q, nk, nv = layers[l]
             if args.fused:
-                hip.decode_layer(q, k, v, sink, hi, recent, budget, scores, idx, out, ws_layer, nk, nv,
-                                 mode=mode, order=hip.ORDER_ANY)
+                hip.decode_layer(q, k, v, sink, hi, recent, budget, scores if args.dense else None, idx,
+                                 out, ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY)
                 continue
-            hist.zero_()
+            if args.dense:
+                hist.zero_()
+            else:
+                hip.select_state_init(n_units, region, budget, ws_sel)
             if ev is not None:
                 ev[4 * l + 0].record()
-            hip.score(k, q, lo, region, mode, q_group=grp, scores=scores, hist=hist)
+            if args.dense:
+                hip.score(k, q, lo, region, mode, q_group=grp, scores=scores, hist=hist)
+            else:
+                hip.score_prune(k, q, lo, region, budget, ws_sel, mode, q_group=grp)
             if ev is not None:
                 ev[4 * l + 1].record()
-            hip.topk_select(scores, budget, mode, hip.ORDER_ANY, hist=hist, idx_out=idx,
-                            workspace=ws_topk)
+            if args.dense:
+                hip.topk_select(scores, budget, mode, hip.ORDER_ANY, hist=hist, idx_out=idx,
+                                workspace=ws_topk)
+            else:
+                hip.sparse_select(idx, n_units, region, budget, ws_sel, mode, hip.ORDER_ANY)
             if ev is not None:
                 ev[4 * l + 2].record()
             hip.gather_attn(q, k, v, idx, k_eff, lo, sink, hi, recent, nk, nv, out=out,
@@ -212,7 +225,7 @@ def main() -> int:
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     score_bytes = n_units * region * hd * 2          # K rows streamed by one score launch
     roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
-                "traffic": None, "kernel": "score_kernel<128>",
+                "traffic": None, "kernel": "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
                 "algorithmic_bytes_per_launch": score_bytes}
     if score_ms is not None:
         ach = score_bytes / (score_ms * 1e-3) / 1e9
@@ -232,7 +245,9 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": cfg["desc"], "key_mode": args.mode,
-                   "call_path": "dc_decode_layer" if args.fused else "dc_score/dc_topk_select/dc_gather_attn"},
+                   "call_path": ("dc_decode_layer" if args.fused else
+                                 "dc_score_bf16/dc_topk_select/dc_gather_attn_bf16" if args.dense else
+                                 "dc_select_state_init/dc_score_prune_bf16/dc_sparse_select/dc_gather_attn_bf16")},
         "step_hbm_gbps": step_gbps,
         "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
         "step_algorithmic_bytes": step_bytes,

@@ -30,6 +30,8 @@ SYMBOLS = (
     "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_append_kv_bf16",
     "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
+    "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
+    "dc_sparse_select", "dc_score_select_bf16",
 )
 
 
@@ -75,6 +77,11 @@ def _load() -> C.CDLL:
         "dc_pq_adc_scan": (i, [p, p, p, p, i, i, i, i64, p]),
         "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
         "dc_compose_idx": (i, [p, i64, p, i64, p, i64, i, i, p]),
+        "dc_score_select_workspace_bytes": (sz, [i, i, i]),
+        "dc_select_state_init": (i, [i, i, i, p, sz, p]),
+        "dc_score_prune_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i, i, i, p, sz, p]),
+        "dc_sparse_select": (i, [p, i64, i, i, i, i, i, i, p, sz, p]),
+        "dc_score_select_bf16": (i, [p, p, p, i64, i, i, i, i, i64, i64, i64, i, i, i, i, p, sz, p]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -179,6 +186,59 @@ def topk_select(scores: torch.Tensor, k: int, mode: int = MODE_REF_DIST, order: 
     return idx_out[:, :k_eff]
 
 
+def score_select_workspace_bytes(n_units: int, n_rows: int, budget: int) -> int:
+    return int(lib.dc_score_select_workspace_bytes(n_units, n_rows, budget))
+
+
+def _score_select_args(store_k, q, lo, n_rows, q_group):
+    sb, sh, sr = _store_strides(store_k)
+    b, h, n_max, hd = store_k.shape
+    if lo < 0 or lo + n_rows > n_max:
+        raise DiffCacheError(f"rows [{lo}, {lo + n_rows}) outside the store of {n_max} rows")
+    if q.dtype != torch.bfloat16 or not q.is_contiguous() or q.numel() != b * h * q_group * hd:
+        raise DiffCacheError("q must be contiguous bf16 with b*h*q_group*hd elements")
+    return _dev(store_k, "store_k") + lo * sr * 2, b, h, hd, sb, sh, sr
+
+
+def select_state_init(n_units: int, n_rows: int, budget: int, workspace: torch.Tensor) -> None:
+    _check(lib.dc_select_state_init(n_units, n_rows, budget, _dev(workspace, "workspace"),
+                                    workspace.numel(), _stream()))
+
+
+def score_prune(store_k: torch.Tensor, q: torch.Tensor, lo: int, n_rows: int, budget: int,
+                workspace: torch.Tensor, mode: int = MODE_REF_DIST, q_group: int = 1) -> None:
+    kptr, b, h, hd, sb, sh, sr = _score_select_args(store_k, q, lo, n_rows, q_group)
+    _check(lib.dc_score_prune_bf16(kptr, _dev(q, "q"), b, h, n_rows, hd, sb, sh, sr, q_group, budget,
+                                   mode, _dev(workspace, "workspace"), workspace.numel(), _stream()))
+
+
+def sparse_select(idx_out: torch.Tensor, n_units: int, n_rows: int, budget: int,
+                  workspace: torch.Tensor, mode: int = MODE_REF_DIST, order: int = ORDER_ANY,
+                  reinit: bool = False) -> torch.Tensor:
+    _check(lib.dc_sparse_select(_dev(idx_out, "idx_out"), idx_out.stride(0), n_units, n_rows, budget,
+                                mode, order, int(reinit), _dev(workspace, "workspace"),
+                                workspace.numel(), _stream()))
+    return idx_out[:, :min(budget, n_rows)]
+
+
+def score_select(store_k: torch.Tensor, q: torch.Tensor, lo: int, n_rows: int, budget: int,
+                 mode: int = MODE_REF_DIST, order: int = ORDER_ANY, q_group: int = 1,
+                 idx_out: Optional[torch.Tensor] = None,
+                 workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Streaming score + exact top-k (no dense scores).  Returns int32 ids
+    (b*h, min(budget, n_rows)) relative to row `lo`."""
+    kptr, b, h, hd, sb, sh, sr = _score_select_args(store_k, q, lo, n_rows, q_group)
+    k_eff = min(budget, n_rows)
+    if idx_out is None:
+        idx_out = torch.empty((b * h, max(k_eff, 1)), dtype=torch.int32, device=store_k.device)
+    if workspace is None:
+        workspace = alloc_workspace(score_select_workspace_bytes(b * h, n_rows, budget), store_k.device)
+    _check(lib.dc_score_select_bf16(kptr, _dev(q, "q"), _dev(idx_out, "idx_out"), idx_out.stride(0), b, h,
+                                    n_rows, hd, sb, sh, sr, q_group, budget, mode, order,
+                                    _dev(workspace, "workspace"), workspace.numel(), _stream()))
+    return idx_out[:, :k_eff]
+
+
 def gather_rows(store_k: Optional[torch.Tensor], store_v: Optional[torch.Tensor], idx: torch.Tensor,
                 out_k: Optional[torch.Tensor], out_v: Optional[torch.Tensor], row_offset: int = 0,
                 n_idx: Optional[int] = None) -> None:
@@ -261,7 +321,7 @@ def layer_workspace_bytes(n_units: int, n_region: int, budget: int, group: int, 
 
 
 def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, n_sink: int,
-                 recent_lo: int, n_recent: int, budget: int, scores: torch.Tensor,
+                 recent_lo: int, n_recent: int, budget: int, scores: Optional[torch.Tensor],
                  idx_out: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor,
                  new_k: Optional[torch.Tensor] = None, new_v: Optional[torch.Tensor] = None,
                  lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
@@ -280,10 +340,11 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
     a.q, a.k, a.v = _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v")
     a.new_k, a.new_v = _opt(new_k, "new_k"), _opt(new_v, "new_v")
     a.out, a.lse = _dev(out, "out"), _opt(lse, "lse")
-    a.scores, a.idx_out = _dev(scores, "scores"), _dev(idx_out, "idx_out")
+    a.scores, a.idx_out = _opt(scores, "scores"), _dev(idx_out, "idx_out")
     a.workspace, a.workspace_bytes = _dev(workspace, "workspace"), workspace.numel()
     a.kv_batch_stride, a.kv_head_stride, a.kv_row_stride = sb, sh, sr
-    a.scores_unit_stride, a.idx_unit_stride = scores.stride(0), idx_out.stride(0)
+    a.scores_unit_stride = 0 if scores is None else scores.stride(0)
+    a.idx_unit_stride = idx_out.stride(0)
     a.recent_lo = recent_lo
     a.n_b, a.n_h, a.group, a.hd = b, h, group, hd
     a.n_sink, a.n_recent, a.budget = n_sink, n_recent, budget

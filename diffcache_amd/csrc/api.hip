@@ -40,7 +40,11 @@ LayerWs carve_layer(void *base, int n_units, int n_region, int budget, int group
     w.hist = (uint32_t *)(p + off);
     off += dc_align_up((size_t)(n_units > 0 ? n_units : 0) * DC_HIST_BINS * 4, 256);
     w.topk = p + off;
-    w.topk_bytes = dc_align_up(dc_topk_workspace_bytes(n_units, n_region, budget), 256);
+    {   // room for either select path: dense scores + dc_topk_select, or the streaming one
+        size_t a = dc_topk_workspace_bytes(n_units, n_region, budget);
+        size_t b = dc_score_select_workspace_bytes(n_units, n_region, budget);
+        w.topk_bytes = dc_align_up(a > b ? a : b, 256);
+    }
     off += w.topk_bytes;
     w.attn = p + off;
     w.attn_bytes = dc_align_up(dc_attn_workspace_bytes(n_units, group, hd, n_attended), 256);
@@ -58,8 +62,7 @@ extern "C" size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int b
 
 extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     DC_REQUIRE(a, "dc_decode_layer: null args");
-    DC_REQUIRE(a->q && a->k && a->v && a->out && a->scores && a->idx_out,
-               "dc_decode_layer: null pointer in args");
+    DC_REQUIRE(a->q && a->k && a->v && a->out && a->idx_out, "dc_decode_layer: null pointer in args");
     DC_REQUIRE(a->n_b >= 0 && a->n_h >= 1 && a->group >= 1 && a->n_sink >= 0 && a->n_recent >= 0 &&
                    a->budget >= 0,
                "dc_decode_layer: bad sizes");
@@ -82,12 +85,18 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     }
     hipStream_t st = (hipStream_t)stream;
     int rc;
-    if (k_eff > 0) {
+    const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
+    if (k_eff > 0 && !a->scores) {
+        // no dense scores wanted: streaming score + select
+        rc = dc_score_select_bf16(k_region, a->q, a->idx_out, a->idx_unit_stride, a->n_b, a->n_h, region,
+                                  a->hd, a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride,
+                                  a->group, a->budget, a->mode, a->order, w.topk, w.topk_bytes, stream);
+        if (rc) return rc;
+    } else if (k_eff > 0) {
         const int64_t n = (int64_t)n_units * DC_HIST_BINS;
         hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                            w.hist, n);
         DC_CHECK_LAUNCH("dc_decode_layer(zero)");
-        const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
         rc = dc_score_bf16(k_region, a->q, a->scores, w.hist, a->n_b, a->n_h, region, a->hd,
                            a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride,
                            a->scores_unit_stride, a->group, a->mode, stream);

@@ -28,6 +28,11 @@ void dc_set_error(const char *fmt, ...);
         }                                                                  \
     } while (0)
 
+// select.hip: sort the selected ids of every unit (see the definition)
+int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t *sel_keys,
+                     uint32_t *idx_out, int64_t idx_stride, unsigned long long *scratch, int n_units,
+                     int k_eff, int mode, int order, hipStream_t st);
+
 static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -104,4 +109,55 @@ __device__ __forceinline__ float dc_dot8(const uint4 &w, const float (&q)[8], fl
     acc = fmaf(dc_bf16_lo(w.w), q[6], acc);
     acc = fmaf(dc_bf16_hi(w.w), q[7], acc);
     return acc;
+}
+
+// This lane's 8 query values (columns col*8 .. col*8+7) of one unit.  A GQA
+// group (q_group > 1) is averaged in fp32 in ascending head order, divided once
+// and rounded to bf16, as torch's bf16 mean does (diffcache.py:193).  The loads
+// of up to 8 heads are issued together; a serial loop covers larger groups.
+template <int HD>
+__device__ __forceinline__ void dc_load_query(const uint16_t *__restrict__ Q, int64_t unit,
+                                              int q_group, int col, float (&q)[8]) {
+    const uint16_t *qp = Q + unit * q_group * HD + col * 8;
+    uint4 raw[8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        raw[g] = make_uint4(0u, 0u, 0u, 0u);
+        if (g < q_group) raw[g] = *reinterpret_cast<const uint4 *>(qp + (int64_t)g * HD);
+    }
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        if (g < q_group) {
+            acc[0] += dc_bf16_lo(raw[g].x);
+            acc[1] += dc_bf16_hi(raw[g].x);
+            acc[2] += dc_bf16_lo(raw[g].y);
+            acc[3] += dc_bf16_hi(raw[g].y);
+            acc[4] += dc_bf16_lo(raw[g].z);
+            acc[5] += dc_bf16_hi(raw[g].z);
+            acc[6] += dc_bf16_lo(raw[g].w);
+            acc[7] += dc_bf16_hi(raw[g].w);
+        }
+    }
+    for (int g = 8; g < q_group; ++g) {
+        const uint4 r = *reinterpret_cast<const uint4 *>(qp + (int64_t)g * HD);
+        acc[0] += dc_bf16_lo(r.x);
+        acc[1] += dc_bf16_hi(r.x);
+        acc[2] += dc_bf16_lo(r.y);
+        acc[3] += dc_bf16_hi(r.y);
+        acc[4] += dc_bf16_lo(r.z);
+        acc[5] += dc_bf16_hi(r.z);
+        acc[6] += dc_bf16_lo(r.w);
+        acc[7] += dc_bf16_hi(r.w);
+    }
+    if (q_group == 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = acc[i];
+    } else {
+        const float n = (float)q_group;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = dc_bf16_to_f32(dc_f32_to_bf16(acc[i] / n));
+    }
 }

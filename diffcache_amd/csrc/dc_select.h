@@ -1,0 +1,157 @@
+// Block-level scan and radix-select helpers shared by the select kernels.
+#pragma once
+#include "dc_common.h"
+
+namespace {
+
+constexpr int kFinalThreads = 1024;
+constexpr int kRadixBits = 11;
+constexpr int kRadixBins = 1 << kRadixBits;
+
+// inclusive scan over the lanes of a wave
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        uint32_t t = __shfl_up(v, d, 64);
+        if (lane >= d) v += t;
+    }
+    return v;
+}
+
+// Block-wide exclusive scan for NT threads (NT a multiple of 64, <= 1024).
+// `wtot` is LDS scratch of at least NT/64 + 1 words.  Returns the exclusive
+// prefix; *total receives the block sum.  Contains two barriers.
+template <int NT>
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, uint32_t *total) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int NW = NT / 64;
+    uint32_t incl = wave_incl_scan(v, lane);
+    if (lane == 63) wtot[wave] = incl;
+    __syncthreads();
+    uint32_t off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        uint32_t t = wtot[w];
+        if (w < wave) off += t;
+        tot += t;
+    }
+    __syncthreads();
+    *total = tot;
+    return off + incl - v;
+}
+
+// Among `n` values v(i), find the rem-th smallest (1-based) by radix passes over
+// bits [hb, 0].  get(i, &value) returns false for items outside the subset.
+// Returns the threshold value; *rem_out = how many items equal to it are needed
+// (rank of the threshold inside its tie group), *n_eq = size of the tie group.
+template <typename Get>
+__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int hb, uint32_t common,
+                                       uint32_t *lh, uint32_t *wtot, uint32_t *sres,
+                                       uint32_t *rem_out, uint32_t *n_eq) {
+    const int tid = threadIdx.x;
+    uint32_t prefix = common;  // bits above hb, shared by every item
+    int top = hb + 1;          // bits [top-1, 0] still undecided
+    uint32_t eq = n;
+    while (top > 0) {
+        const int width = top < kRadixBits ? top : kRadixBits;
+        const int shift = top - width;
+        for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
+        __syncthreads();
+        const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
+        for (uint32_t i = tid; i < n; i += kFinalThreads) {
+            uint32_t v;
+            if (get(i, &v) && ((v & himask) == (prefix & himask)))
+                atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
+        }
+        __syncthreads();
+        // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
+        const uint32_t h0 = lh[2 * tid], h1 = lh[2 * tid + 1];
+        uint32_t total;
+        const uint32_t excl = block_excl_scan<kFinalThreads>(h0 + h1, wtot, &total);
+        if (excl < rem && rem <= excl + h0 + h1) {
+            if (excl + h0 >= rem) {
+                sres[0] = 2 * tid;
+                sres[1] = excl;
+                sres[2] = h0;
+            } else {
+                sres[0] = 2 * tid + 1;
+                sres[1] = excl + h0;
+                sres[2] = h1;
+            }
+        }
+        __syncthreads();
+        prefix |= sres[0] << shift;
+        rem -= sres[1];
+        eq = sres[2];
+        top = shift;
+        __syncthreads();
+    }
+    *rem_out = rem;
+    *n_eq = eq;
+    return prefix;
+}
+
+// Choose the `need` smallest (key, id) pairs among n_c candidates and write
+// their ids to io[0, need).  Must be called by all kFinalThreads threads of a
+// block with uniform arguments.  lh: kRadixBins words, wtot: kFinalThreads/64+1
+// words, sres: 4 words, smisc: 2 words of LDS.  kout (optional) receives the
+// key of each id written.
+__device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_t n_c, uint32_t need,
+                                 uint32_t *io, int n_rows, uint32_t *lh, uint32_t *wtot,
+                                 uint32_t *sres, uint32_t *smisc, uint32_t *kout = nullptr) {
+    const int tid = threadIdx.x;
+    if (need == n_c) {  // the whole candidate list is selected
+        for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
+            io[i] = ci[i];
+            if (kout) kout[i] = ck[i];
+        }
+        return;
+    }
+    // bits in which the candidate keys differ
+    if (tid == 0) {
+        smisc[0] = 0;  // OR of key differences
+        smisc[1] = 0;  // output slot counter
+    }
+    __syncthreads();
+    const uint32_t k0 = ck[0];
+    uint32_t diff = 0;
+    for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
+    if (diff) atomicOr(&smisc[0], diff);
+    __syncthreads();
+    diff = smisc[0];
+    const int hb = diff ? 31 - __clz(diff) : -1;
+    const uint32_t common = (hb >= 31) ? 0u : (k0 & (0xffffffffu << (hb + 1)));
+
+    uint32_t need_eq, n_eq;
+    auto get_key = [&](uint32_t i, uint32_t *v) {
+        *v = ck[i];
+        return true;
+    };
+    const uint32_t t_key =
+        block_radix_select(get_key, n_c, need, hb, common, lh, wtot, sres, &need_eq, &n_eq);
+
+    uint32_t t_idx = 0xffffffffu;
+    if (need_eq < n_eq) {  // only the lowest ids of the tie group fit
+        const uint32_t span = (uint32_t)(n_rows - 1) | 1u;
+        const int hbi = 31 - __clz(span);
+        auto get_idx = [&](uint32_t i, uint32_t *v) {
+            *v = ci[i];
+            return ck[i] == t_key;
+        };
+        uint32_t r2, e2;
+        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi, 0u, lh, wtot, sres, &r2, &e2);
+    }
+
+    for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
+        const uint32_t key = ck[i], id = ci[i];
+        if (key < t_key || (key == t_key && id <= t_idx)) {
+            uint32_t slot = atomicAdd(&smisc[1], 1u);
+            if (slot < need) {
+                io[slot] = id;
+                if (kout) kout[slot] = key;
+            }
+        }
+    }
+}
+
+}  // namespace

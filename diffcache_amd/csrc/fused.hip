@@ -1,0 +1,469 @@
+// Streaming score + exact top-k in two kernels, without a dense score array.
+// Same result as dc_score_bf16 followed by dc_topk_select (the set a size-k heap
+// scan keeps, diffcache_cpu/src/nsw.rs:600-621), built for the case where the
+// scores themselves are not wanted.
+//
+// Why: on MI355X every byte the scan writes costs several read bytes' worth of
+// HBM time, so the 4 bytes/row of a dense score array are the main overhead of
+// a kernel that otherwise streams 256 bytes/row at the read ceiling.
+//
+// score_prune_kernel streams the key rows like score_kernel, bins every key in
+// the unit's 4096-bucket histogram, and keeps a row only if its bucket is not
+// worse than the unit's running threshold bucket tb_run.  tb_run is the bucket
+// of the k-th best key among the rows histogrammed so far; rows can only be
+// added, so tb_run never undershoots the final threshold bucket and no member
+// of the final top-k is ever dropped, however stale the value a block reads.
+// Survivors are staged in LDS and appended to the unit's list as (id, score)
+// with one atomic per block.  Blocks are ordered chunk-major so that all units
+// advance together, and the first chunks of every unit are small so that a
+// threshold exists early.
+//
+// sparse_select_kernel (one block per unit) derives the exact threshold bucket
+// from the complete histogram, splits the survivors into certain members and
+// candidates, and finishes with the same radix select as finalize_kernel.
+#include "dc_common.h"
+#include "dc_select.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRowsPerBlockStep = 256;
+constexpr int kBigSteps = 8;       // 2048 rows per large block
+constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
+constexpr int kStage = kBigSteps * kRowsPerBlockStep;
+
+// tb_run is polled by every wave of the scan while ticket / surv_cnt take
+// returning atomics; they sit in separate 128-byte lines because polling a
+// line that is being updated atomically serialises both at the memory side.
+struct UnitState {
+    uint32_t tb_run;    // running threshold bucket (only decreases)
+    uint32_t pad0[31];
+    uint32_t ticket;    // blocks of this unit that have flushed their histogram
+    uint32_t surv_cnt;  // survivors appended so far
+    uint32_t pad1[30];
+};
+
+__global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t n_hist = (int64_t)n_units * DC_HIST_BINS;
+    if (i < n_hist) hist[i] = 0;
+    if (i < n_units) {
+        state[i].tb_run = DC_HIST_BINS;  // nothing is pruned until a threshold exists
+        state[i].ticket = 0;
+        state[i].surv_cnt = 0;
+    }
+}
+
+__device__ __forceinline__ uint32_t load_relaxed(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int HD>
+__global__ __launch_bounds__(kThreads) void score_prune_kernel(
+    const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, uint32_t *__restrict__ hist,
+    UnitState *__restrict__ state, uint2 *__restrict__ surv, int n_units, int n_h, int n_rows,
+    int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int small_chunks) {
+    constexpr int LPR = HD / 8;
+    constexpr int CH = LPR < 16 ? LPR : 16;
+    __shared__ uint32_t lhist[DC_HIST_BINS];
+    __shared__ uint2 stage[kStage];
+    __shared__ uint32_t wtot[kThreads / 64 + 1];
+    __shared__ uint32_t s_cnt, s_base, s_ticket;
+
+    const int unit = blockIdx.x % n_units;
+    const int chunk = blockIdx.x / n_units;
+    const int b = unit / n_h, h = unit % n_h;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int grp = lane / LPR, col = lane % LPR;
+
+    const bool small = chunk < small_chunks;
+    const int64_t block_row0 =
+        small ? (int64_t)chunk * kRowsPerBlockStep
+              : (int64_t)small_chunks * kRowsPerBlockStep +
+                    (int64_t)(chunk - small_chunks) * kBigSteps * kRowsPerBlockStep;
+    const int steps = small ? 1 : kBigSteps;
+
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
+    if (tid == 0) s_cnt = 0;
+
+    float q[8];
+    dc_load_query<HD>(Q, unit, q_group, col, q);
+    __syncthreads();
+
+    const uint16_t *Ku = K + b * sb + h * sh + col * 8;
+    UnitState *st = state + unit;
+    const int last = n_rows - 1;
+
+    for (int step = 0; step < steps; ++step) {
+        const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
+        if (row0 >= n_rows) break;  // wave-uniform; no barrier inside the loop
+        const uint32_t tb = load_relaxed(&st->tb_run);
+        float mine = 0.f;
+#pragma unroll
+        for (int c0 = 0; c0 < LPR; c0 += CH) {
+            uint4 w[CH];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                int64_t r = row0 + grp * LPR + c0 + j;
+                r = r > last ? last : r;
+                w[j] = *reinterpret_cast<const uint4 *>(Ku + r * sr);
+            }
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                float p = dc_group_sum<LPR>(dc_dot8(w[j], q, 0.f));
+                mine = (col == c0 + j) ? p : mine;
+            }
+        }
+        const int64_t myrow = row0 + lane;
+        const bool valid = myrow < n_rows;
+        uint32_t key = 0, bucket = 0xffffffffu;
+        if (valid) dc_key_bucket(mine, mode, key, bucket);
+        // Only rows that can still matter are kept and counted: the final threshold
+        // bucket is never worse than tb, so it is fixed by the counts of buckets <= tb.
+        const bool keep = valid && bucket <= tb;
+        if (keep) atomicAdd(&lhist[bucket], 1u);
+        const unsigned long long mask = __ballot(keep);
+        if (mask) {
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&s_cnt, (uint32_t)__popcll(mask));
+            base = __shfl(base, 0, 64);
+            if (keep) {
+                const uint32_t pos = base + __popcll(mask & ((1ull << lane) - 1ull));
+                stage[pos] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+            }
+        }
+    }
+    __syncthreads();
+
+    // append this block's survivors to the unit's list
+    const uint32_t cnt = s_cnt;
+    if (tid == 0) s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
+    __syncthreads();
+    {
+        uint2 *dst = surv + (int64_t)unit * n_rows + s_base;
+        for (uint32_t i = tid; i < cnt; i += kThreads) dst[i] = stage[i];
+    }
+    // add the block's histogram to the unit's
+    uint32_t *hu = hist + (int64_t)unit * DC_HIST_BINS;
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
+        const uint32_t c = lhist[i];
+        if (c) atomicAdd(&hu[i], c);
+    }
+    __syncthreads();
+    if (tid == 0) s_ticket = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    // A few blocks per unit refresh the running threshold: every 4th of the
+    // first 32 to finish, then every 8th.  Staleness only loosens the bound.
+    const uint32_t ticket = s_ticket;
+    const bool refresh = ticket < 32u ? (ticket & 3u) == 3u : (ticket & 7u) == 7u;
+    if (!refresh) return;
+
+    // Coalesced, L2-bypassing read of the unit's histogram into LDS (lhist is
+    // free again), then 16 adjacent bins per thread.
+    {
+        const unsigned long long *h64 = reinterpret_cast<const unsigned long long *>(hu);
+        unsigned long long *l64 = reinterpret_cast<unsigned long long *>(lhist);
+        for (int i = tid; i < DC_HIST_BINS / 2; i += kThreads)
+            l64[i] = __hip_atomic_load(h64 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    uint32_t bins[16];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        bins[i] = lhist[tid * 16 + i];
+        sum += bins[i];
+    }
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
+    const uint32_t kk = (uint32_t)k_eff;
+    if (excl < kk && kk <= excl + sum) {
+        uint32_t run = excl;
+        bool done = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (!done && run + bins[i] >= kk) {
+                atomicMin(&st->tb_run, (uint32_t)(tid * 16 + i));
+                done = true;
+            }
+            run += bins[i];
+        }
+    }
+}
+
+// One block per unit: exact threshold bucket from the complete histogram, then
+// certain members / candidates from the survivor list, then the radix select.
+__global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
+    uint32_t *__restrict__ hist, UnitState *__restrict__ state, const uint2 *__restrict__ surv,
+    uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out,
+    int64_t idx_stride, uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int mode, int reinit) {
+    __shared__ uint32_t lh[kRadixBins];
+    __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
+    __shared__ uint32_t sres[4];
+    __shared__ uint32_t smisc[2];
+    __shared__ uint32_t s_tb, s_cless, s_win, s_cand;
+    const int unit = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        s_tb = DC_HIST_BINS;
+        s_cless = 0;
+        s_win = 0;
+        s_cand = 0;
+    }
+    uint32_t bins[4];
+    {
+        const uint4 t = reinterpret_cast<const uint4 *>(hist + (int64_t)unit * DC_HIST_BINS)[tid];
+        // (each thread re-zeroes exactly the four bins it read, see the end of the survivor loop)
+        bins[0] = t.x;
+        bins[1] = t.y;
+        bins[2] = t.z;
+        bins[3] = t.w;
+    }
+    const uint32_t sum = bins[0] + bins[1] + bins[2] + bins[3];
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<kFinalThreads>(sum, wtot, &total);
+    const uint32_t kk = (uint32_t)k_eff;
+    if (excl < kk && kk <= excl + sum) {
+        uint32_t run = excl;
+        bool done = false;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (!done && run + bins[i] >= kk) {
+                s_tb = tid * 4 + i;
+                s_cless = run;
+                done = true;
+            }
+            run += bins[i];
+        }
+    }
+    __syncthreads();
+    const uint32_t tb = s_tb, c_less = s_cless;
+    uint32_t n_s = state[unit].surv_cnt;
+    if (n_s > (uint32_t)n_rows) n_s = n_rows;
+    const uint2 *su = surv + (int64_t)unit * n_rows;
+    uint32_t *ck = cand_key + (int64_t)unit * n_rows;
+    uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride;
+    uint32_t *ko = sel_keys ? sel_keys + (int64_t)unit * k_eff : nullptr;
+
+    const int lane = tid & 63;
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    for (uint32_t i0 = 0; i0 < n_s; i0 += kFinalThreads) {
+        const uint32_t i = i0 + tid;
+        uint32_t key = 0, bucket = 0xffffffffu, id = 0;
+        if (i < n_s) {
+            const uint2 p = su[i];
+            id = p.x;
+            dc_key_bucket(__uint_as_float(p.y), mode, key, bucket);
+        }
+        // one LDS atomic per wave and list
+        const bool is_win = bucket < tb, is_cand = bucket == tb;
+        const unsigned long long mw = __ballot(is_win), mc = __ballot(is_cand);
+        if (mw) {
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&s_win, (uint32_t)__popcll(mw));
+            base = __shfl(base, 0, 64);
+            const uint32_t slot = base + __popcll(mw & lt);
+            if (is_win && slot < kk) {
+                io[slot] = id;
+                if (ko) ko[slot] = key;
+            }
+        }
+        if (mc) {
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&s_cand, (uint32_t)__popcll(mc));
+            base = __shfl(base, 0, 64);
+            const uint32_t slot = base + __popcll(mc & lt);
+            if (is_cand && slot < (uint32_t)n_rows) {
+                ck[slot] = key;
+                ci[slot] = id;
+            }
+        }
+    }
+    __syncthreads();
+    if (reinit) {
+        // leave the unit's histogram and counters ready for the next scan
+        uint4 *hz = reinterpret_cast<uint4 *>(hist + (int64_t)unit * DC_HIST_BINS);
+        hz[tid] = make_uint4(0u, 0u, 0u, 0u);
+        if (tid == 0) {
+            state[unit].tb_run = DC_HIST_BINS;
+            state[unit].ticket = 0;
+            state[unit].surv_cnt = 0;
+        }
+    }
+    uint32_t n_c = s_cand;
+    if (n_c > (uint32_t)n_rows) n_c = n_rows;
+    if (c_less >= kk) return;
+    uint32_t need = kk - c_less;
+    if (need > n_c) need = n_c;
+    dc_finalize_unit(ck, ci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc,
+                     ko ? ko + c_less : nullptr);
+}
+
+struct FusedWs {
+    uint32_t *hist;
+    UnitState *state;
+    uint2 *surv;
+    uint32_t *cand_key, *cand_idx, *sel_keys;
+    unsigned long long *sort_scratch;
+    size_t bytes;
+};
+
+int fused_pow2(int x) {
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+FusedWs carve_fused(void *base, int n_units, int n_rows, int k) {
+    FusedWs w;
+    char *p = (char *)base;
+    size_t off = 0;
+    const size_t nu = n_units > 0 ? n_units : 0, nr = n_rows > 0 ? n_rows : 0;
+    const int keff = k < n_rows ? k : n_rows;
+    w.hist = (uint32_t *)(p + off);
+    off += dc_align_up(nu * DC_HIST_BINS * 4, 256);
+    w.state = (UnitState *)(p + off);
+    off += dc_align_up(nu * sizeof(UnitState), 256);
+    w.surv = (uint2 *)(p + off);
+    off += dc_align_up(nu * nr * 8, 256);
+    w.cand_key = (uint32_t *)(p + off);
+    off += dc_align_up(nu * nr * 4, 256);
+    w.cand_idx = (uint32_t *)(p + off);
+    off += dc_align_up(nu * nr * 4, 256);
+    w.sel_keys = (uint32_t *)(p + off);
+    off += dc_align_up(nu * (size_t)(keff > 0 ? keff : 0) * 4, 256);
+    w.sort_scratch = (unsigned long long *)(p + off);
+    if (keff > 4096) off += dc_align_up(nu * (size_t)fused_pow2(keff) * 8, 256);
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k) {
+    return carve_fused(nullptr, n_units, n_rows, k).bytes;
+}
+
+namespace {
+
+struct FusedPlan {
+    int n_units, k_eff, small_chunks;
+    int64_t blocks;
+};
+
+int plan_fused(const char *who, int n_b, int n_h, int n_rows, int budget, FusedPlan *p) {
+    DC_REQUIRE(n_b >= 0 && n_h >= 1 && n_rows >= 0 && budget >= 0, "%s: bad sizes", who);
+    const int64_t n_units64 = (int64_t)n_b * n_h;
+    DC_REQUIRE(n_units64 < (1 << 20), "%s: too many units", who);
+    p->n_units = (int)n_units64;
+    p->k_eff = budget < n_rows ? budget : n_rows;
+    // chunks per unit: up to kSmallChunks blocks of 256 rows, then blocks of 2048 rows
+    const int64_t tiles = ((int64_t)n_rows + kRowsPerBlockStep - 1) / kRowsPerBlockStep;
+    p->small_chunks = (int)(tiles < kSmallChunks ? tiles : kSmallChunks);
+    const int64_t rest = (int64_t)n_rows - (int64_t)p->small_chunks * kRowsPerBlockStep;
+    const int64_t big_chunks = rest > 0 ? (rest + kStage - 1) / kStage : 0;
+    p->blocks = n_units64 * (p->small_chunks + big_chunks);
+    DC_REQUIRE(p->blocks < (1ll << 31), "%s: grid too large", who);
+    return DC_OK;
+}
+
+int check_ws(const char *who, void *workspace, size_t workspace_bytes, int n_units, int n_rows,
+             int budget, FusedWs *w) {
+    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
+               "%s: workspace must be non-null and 256-byte aligned", who);
+    *w = carve_fused(workspace, n_units, n_rows, budget);
+    if (workspace_bytes < w->bytes) {
+        dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, w->bytes);
+        return DC_ENOMEM;
+    }
+    return DC_OK;
+}
+
+}  // namespace
+
+extern "C" int dc_select_state_init(int n_units, int n_rows, int budget, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(n_units >= 0 && n_rows >= 0 && budget >= 0, "dc_select_state_init: bad sizes");
+    if (n_units == 0) return DC_OK;
+    FusedWs w;
+    int rc = check_ws("dc_select_state_init", workspace, workspace_bytes, n_units, n_rows, budget, &w);
+    if (rc) return rc;
+    const int64_t n = (int64_t)n_units * DC_HIST_BINS;
+    hipLaunchKernelGGL(init_state_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, w.hist, w.state, n_units);
+    DC_CHECK_LAUNCH("dc_select_state_init");
+    return DC_OK;
+}
+
+extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_h, int n_rows, int hd,
+                                   int64_t sb, int64_t sh, int64_t sr, int q_group, int budget,
+                                   int mode, void *workspace, size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(k && q, "dc_score_prune_bf16: null pointer");
+    DC_REQUIRE(q_group >= 1, "dc_score_prune_bf16: bad q_group");
+    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "dc_score_prune_bf16: head_dim %d not in {64,128,256}", hd);
+    DC_REQUIRE(mode == DC_MODE_IP || mode == DC_MODE_REF_DIST, "dc_score_prune_bf16: bad mode %d", mode);
+    DC_REQUIRE(dc_aligned16(k), "dc_score_prune_bf16: k must be 16-byte aligned");
+    DC_REQUIRE(sb % 8 == 0 && sh % 8 == 0 && sr % 8 == 0 && sr >= hd,
+               "dc_score_prune_bf16: strides must be multiples of 8 elements and row_stride >= hd");
+    FusedPlan p;
+    int rc = plan_fused("dc_score_prune_bf16", n_b, n_h, n_rows, budget, &p);
+    if (rc) return rc;
+    if (p.n_units == 0 || p.k_eff == 0) return DC_OK;
+    FusedWs w;
+    rc = check_ws("dc_score_prune_bf16", workspace, workspace_bytes, p.n_units, n_rows, budget, &w);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+#define DC_LAUNCH_SP(HD)                                                                           \
+    hipLaunchKernelGGL(score_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st,    \
+                       (const uint16_t *)k, (const uint16_t *)q, w.hist, w.state, w.surv,          \
+                       p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode, p.k_eff, p.small_chunks)
+    if (hd == 64) DC_LAUNCH_SP(64);
+    else if (hd == 128) DC_LAUNCH_SP(128);
+    else DC_LAUNCH_SP(256);
+#undef DC_LAUNCH_SP
+    DC_CHECK_LAUNCH("dc_score_prune_bf16");
+    return DC_OK;
+}
+
+extern "C" int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int n_units, int n_rows,
+                                int budget, int mode, int order, int reinit, void *workspace,
+                                size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(idx_out, "dc_sparse_select: null pointer");
+    DC_REQUIRE(n_units >= 0 && n_rows >= 0 && budget >= 0, "dc_sparse_select: bad sizes");
+    DC_REQUIRE(mode == DC_MODE_IP || mode == DC_MODE_REF_DIST, "dc_sparse_select: bad mode %d", mode);
+    DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "dc_sparse_select: bad order %d", order);
+    const int k_eff = budget < n_rows ? budget : n_rows;
+    if (n_units == 0 || k_eff == 0) return DC_OK;
+    DC_REQUIRE(idx_unit_stride >= k_eff, "dc_sparse_select: idx_unit_stride < min(budget, n_rows)");
+    FusedWs w;
+    int rc = check_ws("dc_sparse_select", workspace, workspace_bytes, n_units, n_rows, budget, &w);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
+    hipLaunchKernelGGL(sparse_select_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.hist, w.state,
+                       w.surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows,
+                       k_eff, mode, reinit);
+    DC_CHECK_LAUNCH("dc_sparse_select");
+    if (order != DC_ORDER_ANY)
+        return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
+                                k_eff, mode, order, st);
+    return DC_OK;
+}
+
+extern "C" int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out,
+                                    int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                                    int64_t sb, int64_t sh, int64_t sr, int q_group, int budget,
+                                    int mode, int order, void *workspace, size_t workspace_bytes,
+                                    void *stream) {
+    DC_REQUIRE(n_b >= 0 && n_h >= 1, "dc_score_select_bf16: bad sizes");
+    const int n_units = n_b * n_h;
+    int rc = dc_select_state_init(n_units, n_rows, budget, workspace, workspace_bytes, stream);
+    if (rc) return rc;
+    rc = dc_score_prune_bf16(k, q, n_b, n_h, n_rows, hd, sb, sh, sr, q_group, budget, mode, workspace,
+                             workspace_bytes, stream);
+    if (rc) return rc;
+    return dc_sparse_select(idx_out, idx_unit_stride, n_units, n_rows, budget, mode, order, 0, workspace,
+                            workspace_bytes, stream);
+}

@@ -48,20 +48,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
     // this lane's 8 query values; a GQA group is averaged in fp32 and rounded to
     // bf16 first (diffcache.py:193)
     float q[8];
-    {
-        const uint16_t *qp = Q + (int64_t)unit * q_group * HD + col * 8;
-        if (q_group == 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) q[i] = dc_bf16_to_f32(qp[i]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float acc = 0.f;
-                for (int g = 0; g < q_group; ++g) acc += dc_bf16_to_f32(qp[(int64_t)g * HD + i]);
-                q[i] = dc_bf16_to_f32(dc_f32_to_bf16(acc / (float)q_group));
-            }
-        }
-    }
+    dc_load_query<HD>(Q, unit, q_group, col, q);
 
     const uint16_t *Ku = K + b * sb + h * sh + col * 8;
     float *su = scores + (int64_t)unit * scores_stride;

@@ -14,15 +14,13 @@
 //      on the 32-bit key, then on the id among keys equal to the threshold.
 // An optional sort_kernel orders the k ids (best first, or by id).
 #include "dc_common.h"
+#include "dc_select.h"
 
 namespace {
 
 constexpr int kFilterThreads = 256;
 constexpr int kFilterPerThread = 32;
 constexpr int kFilterChunk = kFilterThreads * kFilterPerThread;  // 8192 scores per block
-constexpr int kFinalThreads = 1024;
-constexpr int kRadixBits = 11;
-constexpr int kRadixBins = 1 << kRadixBits;
 constexpr int kSortLds = 4096;
 
 struct UnitMeta {
@@ -63,38 +61,6 @@ __global__ __launch_bounds__(kFilterThreads) void hist_kernel(
         uint32_t c = lhist[i];
         if (c) atomicAdd(&hu[i], c);
     }
-}
-
-// inclusive scan over the lanes of a wave
-__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        uint32_t t = __shfl_up(v, d, 64);
-        if (lane >= d) v += t;
-    }
-    return v;
-}
-
-// Block-wide exclusive scan for NT threads (NT a multiple of 64, <= 1024).
-// `wtot` is LDS scratch of at least NT/64 + 1 words.  Returns the exclusive
-// prefix; *total receives the block sum.  Contains two barriers.
-template <int NT>
-__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, uint32_t *total) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    constexpr int NW = NT / 64;
-    uint32_t incl = wave_incl_scan(v, lane);
-    if (lane == 63) wtot[wave] = incl;
-    __syncthreads();
-    uint32_t off = 0, tot = 0;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-        uint32_t t = wtot[w];
-        if (w < wave) off += t;
-        tot += t;
-    }
-    __syncthreads();
-    *total = tot;
-    return off + incl - v;
 }
 
 __global__ __launch_bounds__(kFilterThreads) void filter_kernel(
@@ -197,57 +163,6 @@ __global__ __launch_bounds__(kFilterThreads) void filter_kernel(
     }
 }
 
-// Among `n` values v(i), find the rem-th smallest (1-based) by radix passes over
-// bits [hb, 0].  get(i, &value) returns false for items outside the subset.
-// Returns the threshold value; *rem_out = how many items equal to it are needed
-// (rank of the threshold inside its tie group), *n_eq = size of the tie group.
-template <typename Get>
-__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int hb, uint32_t common,
-                                       uint32_t *lh, uint32_t *wtot, uint32_t *sres,
-                                       uint32_t *rem_out, uint32_t *n_eq) {
-    const int tid = threadIdx.x;
-    uint32_t prefix = common;  // bits above hb, shared by every item
-    int top = hb + 1;          // bits [top-1, 0] still undecided
-    uint32_t eq = n;
-    while (top > 0) {
-        const int width = top < kRadixBits ? top : kRadixBits;
-        const int shift = top - width;
-        for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
-        __syncthreads();
-        const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
-        for (uint32_t i = tid; i < n; i += kFinalThreads) {
-            uint32_t v;
-            if (get(i, &v) && ((v & himask) == (prefix & himask)))
-                atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
-        }
-        __syncthreads();
-        // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
-        const uint32_t h0 = lh[2 * tid], h1 = lh[2 * tid + 1];
-        uint32_t total;
-        const uint32_t excl = block_excl_scan<kFinalThreads>(h0 + h1, wtot, &total);
-        if (excl < rem && rem <= excl + h0 + h1) {
-            if (excl + h0 >= rem) {
-                sres[0] = 2 * tid;
-                sres[1] = excl;
-                sres[2] = h0;
-            } else {
-                sres[0] = 2 * tid + 1;
-                sres[1] = excl + h0;
-                sres[2] = h1;
-            }
-        }
-        __syncthreads();
-        prefix |= sres[0] << shift;
-        rem -= sres[1];
-        eq = sres[2];
-        top = shift;
-        __syncthreads();
-    }
-    *rem_out = rem;
-    *n_eq = eq;
-    return prefix;
-}
-
 __global__ __launch_bounds__(kFinalThreads) void finalize_kernel(
     const UnitMeta *__restrict__ meta, const uint32_t *__restrict__ cand_key,
     const uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out, int64_t idx_stride,
@@ -255,87 +170,38 @@ __global__ __launch_bounds__(kFinalThreads) void finalize_kernel(
     __shared__ uint32_t lh[kRadixBins];
     __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
     __shared__ uint32_t sres[4];
-    __shared__ uint32_t s_diff, s_slot;
+    __shared__ uint32_t smisc[2];
     const int unit = blockIdx.x;
-    const int tid = threadIdx.x;
     const uint32_t c_less = meta[unit].c_less;
     uint32_t n_c = meta[unit].cand_cnt;
     if (n_c > (uint32_t)n_rows) n_c = n_rows;
     if (c_less >= (uint32_t)k_eff) return;
     uint32_t need = (uint32_t)k_eff - c_less;
     if (need > n_c) need = n_c;
-    const uint32_t *ck = cand_key + (int64_t)unit * n_rows;
-    const uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
-    uint32_t *io = idx_out + (int64_t)unit * idx_stride + c_less;
-
-    if (need == n_c) {  // the whole threshold bucket is selected
-        for (uint32_t i = tid; i < n_c; i += kFinalThreads) io[i] = ci[i];
-        return;
-    }
-
-    // bits in which the candidate keys differ
-    if (tid == 0) {
-        s_diff = 0;
-        s_slot = 0;
-    }
-    __syncthreads();
-    const uint32_t k0 = ck[0];
-    uint32_t diff = 0;
-    for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
-    if (diff) atomicOr(&s_diff, diff);
-    __syncthreads();
-    diff = s_diff;
-    const int hb = diff ? 31 - __clz(diff) : -1;
-    const uint32_t common = (hb >= 31) ? 0u : (k0 & (0xffffffffu << (hb + 1)));
-
-    uint32_t need_eq, n_eq;
-    auto get_key = [&](uint32_t i, uint32_t *v) {
-        *v = ck[i];
-        return true;
-    };
-    const uint32_t t_key =
-        block_radix_select(get_key, n_c, need, hb, common, lh, wtot, sres, &need_eq, &n_eq);
-
-    uint32_t t_idx = 0xffffffffu;
-    if (need_eq < n_eq) {  // only the lowest ids of the tie group fit
-        const uint32_t span = (uint32_t)(n_rows - 1) | 1u;
-        const int hbi = 31 - __clz(span);
-        auto get_idx = [&](uint32_t i, uint32_t *v) {
-            *v = ci[i];
-            return ck[i] == t_key;
-        };
-        uint32_t r2, e2;
-        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi, 0u, lh, wtot, sres, &r2, &e2);
-    }
-
-    for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
-        const uint32_t key = ck[i], id = ci[i];
-        if (key < t_key || (key == t_key && id <= t_idx)) {
-            uint32_t slot = atomicAdd(&s_slot, 1u);
-            if (slot < need) io[slot] = id;
-        }
-    }
+    dc_finalize_unit(cand_key + (int64_t)unit * n_rows, cand_idx + (int64_t)unit * n_rows, n_c, need,
+                     idx_out + (int64_t)unit * idx_stride + c_less, n_rows, lh, wtot, sres, smisc);
 }
 
 // Bitonic sort of each unit's k ids by (key, id) or by id.
 template <bool IN_LDS>
 __global__ __launch_bounds__(kFinalThreads) void sort_kernel(
-    const float *__restrict__ scores, int64_t scores_stride, uint32_t *__restrict__ idx_out,
-    int64_t idx_stride, unsigned long long *__restrict__ scratch, int k_eff, int pow2, int mode,
-    int order) {
+    const float *__restrict__ scores, int64_t scores_stride, const uint32_t *__restrict__ sel_keys,
+    uint32_t *__restrict__ idx_out, int64_t idx_stride, unsigned long long *__restrict__ scratch,
+    int k_eff, int pow2, int mode, int order) {
     __shared__ unsigned long long lbuf[IN_LDS ? kSortLds : 1];
     const int unit = blockIdx.x;
     const int tid = threadIdx.x;
     unsigned long long *buf = IN_LDS ? lbuf : scratch + (int64_t)unit * pow2;
     uint32_t *io = idx_out + (int64_t)unit * idx_stride;
-    const float *su = scores + (int64_t)unit * scores_stride;
+    const float *su = scores ? scores + (int64_t)unit * scores_stride : nullptr;
     for (int i = tid; i < pow2; i += kFinalThreads) {
         unsigned long long v = ~0ull;
         if (i < k_eff) {
             uint32_t id = io[i];
             if (order == DC_ORDER_BEST) {
                 uint32_t key, bucket;
-                dc_key_bucket(su[id], mode, key, bucket);
+                if (sel_keys) key = sel_keys[(int64_t)unit * k_eff + i];
+                else dc_key_bucket(su[id], mode, key, bucket);
                 v = ((unsigned long long)key << 32) | id;
             } else {
                 v = id;
@@ -407,6 +273,24 @@ SelectWs carve(void *base, int n_units, int n_rows, int k) {
 
 }  // namespace
 
+// Sort each unit's k_eff selected ids: DC_ORDER_BEST by (key, id) with the key
+// taken from sel_keys (n_units, k_eff) when given, else recomputed from the dense
+// scores; DC_ORDER_INDEX by id.  scratch is needed when k_eff > 4096.
+int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t *sel_keys,
+                     uint32_t *idx_out, int64_t idx_stride, unsigned long long *scratch, int n_units,
+                     int k_eff, int mode, int order, hipStream_t st) {
+    const int p2 = next_pow2(k_eff);
+    if (p2 <= kSortLds)
+        hipLaunchKernelGGL(sort_kernel<true>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
+                           scores_stride, sel_keys, idx_out, idx_stride,
+                           (unsigned long long *)nullptr, k_eff, p2, mode, order);
+    else
+        hipLaunchKernelGGL(sort_kernel<false>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
+                           scores_stride, sel_keys, idx_out, idx_stride, scratch, k_eff, p2, mode, order);
+    DC_CHECK_LAUNCH("dc_sort_selected");
+    return DC_OK;
+}
+
 extern "C" size_t dc_topk_workspace_bytes(int n_units, int n_rows, int k) {
     if (n_units <= 0 || n_rows <= 0 || k <= 0) return 256;
     return carve(nullptr, n_units, n_rows, k).bytes;
@@ -456,18 +340,9 @@ extern "C" int dc_topk_select(const float *scores, int64_t scores_unit_stride, u
     hipLaunchKernelGGL(finalize_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.meta,
                        w.cand_key, w.cand_idx, idx_out, idx_unit_stride, n_rows, k_eff);
     DC_CHECK_LAUNCH("dc_topk_select(finalize)");
-    if (order != DC_ORDER_ANY) {
-        const int p2 = next_pow2(k_eff);
-        if (p2 <= kSortLds)
-            hipLaunchKernelGGL(sort_kernel<true>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
-                               scores_unit_stride, idx_out, idx_unit_stride,
-                               (unsigned long long *)nullptr, k_eff, p2, mode, order);
-        else
-            hipLaunchKernelGGL(sort_kernel<false>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
-                               scores_unit_stride, idx_out, idx_unit_stride, w.sort_scratch, k_eff,
-                               p2, mode, order);
-        DC_CHECK_LAUNCH("dc_topk_select(sort)");
-    }
+    if (order != DC_ORDER_ANY)
+        return dc_sort_selected(scores, scores_unit_stride, nullptr, idx_out, idx_unit_stride,
+                                w.sort_scratch, n_units, k_eff, mode, order, st);
     return DC_OK;
 }
 

@@ -100,6 +100,37 @@ int dc_topk_select(const float *scores, int64_t scores_unit_stride, uint32_t *id
                    const uint32_t *hist, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Streaming score + exact top-k without a dense score array: the same ids as
+ * dc_score_bf16 followed by dc_topk_select (identical arithmetic), for callers
+ * that do not want the scores.  The scan writes only the rows that can still
+ * reach the top-k, which matters because HBM writes are far dearer than reads
+ * on this part.  Arguments as in dc_score_bf16 / dc_topk_select; `budget` is k.
+ * Three steps that may also be called one by one on the same workspace:
+ *   dc_select_state_init   clears the per-unit histogram and counters
+ *   dc_score_prune_bf16    the scan (the HBM-bound kernel)
+ *   dc_sparse_select       exact selection among the surviving rows; with reinit != 0
+ *                          it also leaves the workspace as dc_select_state_init does, so
+ *                          the next dc_score_prune_bf16 of the same sizes on it needs no
+ *                          init call
+ * Replaces the same reference code as the two calls it stands for
+ * (diffcache_cpu/src/nsw.rs:129-139,600-621).
+ */
+size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int budget);
+int dc_select_state_init(int n_units, int n_rows, int budget, void *workspace,
+                         size_t workspace_bytes, void *stream);
+int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_h, int n_rows, int hd,
+                        int64_t k_batch_stride, int64_t k_head_stride, int64_t k_row_stride,
+                        int q_group, int budget, int mode, void *workspace, size_t workspace_bytes,
+                        void *stream);
+int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int n_units, int n_rows, int budget,
+                     int mode, int order, int reinit, void *workspace, size_t workspace_bytes,
+                     void *stream);
+int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out, int64_t idx_unit_stride,
+                         int n_b, int n_h, int n_rows, int hd, int64_t k_batch_stride,
+                         int64_t k_head_stride, int64_t k_row_stride, int q_group, int budget,
+                         int mode, int order, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Copy selected K and V rows into dense output buffers.
  * For unit (b, h) and j < n_idx:
  *   out_k[b, h, j, :] = k[b, h, row_offset + idx[u, j], :]   (same for v)
@@ -175,7 +206,8 @@ typedef struct dc_layer_args {
     const void *new_v;
     void *out;            /* (n_b, n_h*group, hd) bf16 */
     float *lse;           /* (n_b, n_h*group) or NULL */
-    float *scores;        /* (n_units, scores_unit_stride) fp32 scratch/output */
+    float *scores;        /* (n_units, scores_unit_stride) fp32 output, or NULL: scores are
+                             not materialised and the streaming select is used */
     uint32_t *idx_out;    /* (n_units, idx_unit_stride) */
     void *workspace;      /* dc_layer_workspace_bytes(...) bytes, 256-byte aligned */
     size_t workspace_bytes;

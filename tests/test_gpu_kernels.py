@@ -211,6 +211,71 @@ def test_select_property_invariants_1m_rows():
         assert torch.equal(torch.sort(ref_vals, descending=True).values, got)
 
 
+# ------------------------------------------------------------------ streaming score + select
+
+def check_streaming(k_u16, q_u16, lo, n_rows, budget, mode, order, q_group=1):
+    """ids of the streaming path == oracle top-k of the dense scores of the same arithmetic"""
+    store, qd = to_dev_bf16(k_u16), to_dev_bf16(q_u16)
+    dense = hip.score(store, qd, lo, n_rows, mode, q_group=q_group).cpu().numpy()
+    ids = hip.score_select(store, qd, lo, n_rows, budget, mode, order, q_group=q_group)
+    ids = ids.cpu().numpy().astype(np.uint32)
+    k_eff = min(budget, n_rows)
+    for u in range(dense.shape[0]):
+        want = orc.topk_select(dense[u], budget, mode)
+        got = ids[u, :k_eff]
+        if order == hip.ORDER_BEST:
+            assert np.array_equal(got, want), f"unit {u}"
+        elif order == hip.ORDER_INDEX:
+            assert np.array_equal(got, np.sort(want)), f"unit {u}"
+        else:
+            assert np.array_equal(np.sort(got), np.sort(want)), f"unit {u}"
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("hd", [64, 128, 256])
+@pytest.mark.parametrize("n_rows,budget", [(1, 1), (255, 16), (257, 300), (8192, 128), (8193, 1024),
+                                           (30000, 2048)])
+def test_streaming_select_matches_dense_path(mode, hd, n_rows, budget):
+    rng = np.random.default_rng(hd + n_rows + budget + mode)
+    b, h, lo = 2, 2, 3
+    print(f"streaming mode={mode} hd={hd} n_rows={n_rows} budget={budget}", flush=True)
+    k = rand_bf16(rng, b, h, lo + n_rows + 2, hd)
+    q = rand_bf16(rng, b, h, hd)
+    check_streaming(k, q, lo, n_rows, budget, mode, hip.ORDER_BEST)
+    check_streaming(k, q, lo, n_rows, budget, mode, hip.ORDER_ANY)
+
+
+def test_streaming_select_ties_and_group_mean():
+    rng = np.random.default_rng(77)
+    b, h, g, hd, n = 1, 3, 4, 128, 20000
+    # small-integer keys: many exact score ties; zero query for unit 2: everything ties
+    k = orc.f32_to_bf16(rng.integers(-2, 3, (b, h, n, hd)).astype(np.float32))
+    q = orc.f32_to_bf16(rng.integers(-1, 2, (b, h * g, hd)).astype(np.float32))
+    q[0, 2 * g:3 * g] = 0
+    for mode in (0, 1):
+        check_streaming(k, q, 0, n, 1500, mode, hip.ORDER_BEST, q_group=g)
+        check_streaming(k, q, 0, n, 1500, mode, hip.ORDER_INDEX, q_group=g)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_streaming_select_full_size_unit(mode):
+    # benchmark shape: 131004-row region, k 2048, keys with outlier channels; 8 units
+    rng = np.random.default_rng(123 + mode)
+    b, h, hd, n = 1, 8, 128, 131072
+    scale = np.exp(rng.standard_normal((1, h, 1, hd))).astype(np.float32)
+    k = orc.f32_to_bf16(rng.standard_normal((b, h, n, hd)).astype(np.float32) * scale)
+    q = rand_bf16(rng, b, h, hd)
+    check_streaming(k, q, 4, n - 68, 2048, mode, hip.ORDER_BEST)
+
+
+def test_streaming_select_large_budget():
+    rng = np.random.default_rng(5)
+    k = rand_bf16(rng, 1, 2, 40000, 128)
+    q = rand_bf16(rng, 1, 2, 128)
+    check_streaming(k, q, 0, 40000, 9000, hip.MODE_REF_DIST, hip.ORDER_BEST)
+    check_streaming(k, q, 0, 40000, 50000, hip.MODE_IP, hip.ORDER_ANY)
+
+
 # ------------------------------------------------------------------ gather rows / kv maintenance
 
 def test_gather_rows_and_ingest_append():
@@ -326,6 +391,15 @@ def run_layer(rng, b, hq, hkv, n_ctx, hd, budget, p, s, mode, new_tok, n_max=Non
     got = orc.bf16_to_f32(to_np_u16(out))
     sc = scores.cpu().numpy()
     ids = idx.cpu().numpy().astype(np.uint32)
+    # the same layer without a dense score array (streaming select) must pick the same ids
+    idx2 = torch.full_like(idx, -1)
+    out2 = torch.empty_like(out)
+    hip.decode_layer(to_dev_bf16(q), to_dev_bf16(k), to_dev_bf16(v), p_len, hi, s_len, budget,
+                     None, idx2, out2, ws, None if nk is None else to_dev_bf16(nk),
+                     None if nv is None else to_dev_bf16(nv), mode=mode, order=hip.ORDER_BEST)
+    torch.cuda.synchronize()
+    assert np.array_equal(idx2.cpu().numpy()[:, :k_eff], idx.cpu().numpy()[:, :k_eff])
+    assert np.array_equal(to_np_u16(out2), to_np_u16(out))
     for bi in range(b):
         so = sc[bi * hkv:(bi + 1) * hkv, :region]
         res = orc.decode_layer(q[bi], k[bi, :, :n_ctx], v[bi, :, :n_ctx], hkv, budget, p, s, mode,
