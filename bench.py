@@ -166,6 +166,8 @@ def main() -> int:
     def new_events(count):
         return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
 
+    state = {"clean": False}
+
     def step(ev=None):
         """One decode step: every layer, in order, on the current stream."""
         for l in range(L):
@@ -176,8 +178,9 @@ def main() -> int:
                 continue
             if args.dense:
                 hist.zero_()
-            else:
+            elif not state["clean"]:
                 hip.select_state_init(n_units, region, budget, ws_sel)
+                state["clean"] = True   # dc_sparse_select(reinit) keeps it so from here on
             if ev is not None:
                 ev[4 * l + 0].record()
             if args.dense:
@@ -190,7 +193,7 @@ def main() -> int:
                 hip.topk_select(scores, budget, mode, hip.ORDER_ANY, hist=hist, idx_out=idx,
                                 workspace=ws_topk)
             else:
-                hip.sparse_select(idx, n_units, region, budget, ws_sel, mode, hip.ORDER_ANY)
+                hip.sparse_select(idx, n_units, region, budget, ws_sel, mode, hip.ORDER_ANY, reinit=True)
             if ev is not None:
                 ev[4 * l + 2].record()
             hip.gather_attn(q, k, v, idx, k_eff, lo, sink, hi, recent, nk, nv, out=out,

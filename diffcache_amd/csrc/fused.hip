@@ -31,6 +31,7 @@ constexpr int kRowsPerBlockStep = 256;
 constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
+constexpr int kCandLds = 4096;
 
 // tb_run is polled by every wave of the scan while ticket / surv_cnt take
 // returning atomics; they sit in separate 128-byte lines because polling a
@@ -62,7 +63,8 @@ template <int HD>
 __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, uint32_t *__restrict__ hist,
     UnitState *__restrict__ state, uint2 *__restrict__ surv, int n_units, int n_h, int n_rows,
-    int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int small_chunks) {
+    int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int small_chunks,
+    int big_steps) {
     constexpr int LPR = HD / 8;
     constexpr int CH = LPR < 16 ? LPR : 16;
     __shared__ uint32_t lhist[DC_HIST_BINS];
@@ -81,8 +83,8 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     const int64_t block_row0 =
         small ? (int64_t)chunk * kRowsPerBlockStep
               : (int64_t)small_chunks * kRowsPerBlockStep +
-                    (int64_t)(chunk - small_chunks) * kBigSteps * kRowsPerBlockStep;
-    const int steps = small ? 1 : kBigSteps;
+                    (int64_t)(chunk - small_chunks) * big_steps * kRowsPerBlockStep;
+    const int steps = small ? 1 : big_steps;
 
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
     if (tid == 0) s_cnt = 0;
@@ -203,6 +205,7 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
     __shared__ uint32_t sres[4];
     __shared__ uint32_t smisc[2];
     __shared__ uint32_t s_tb, s_cless, s_win, s_cand;
+    __shared__ uint32_t lck[kCandLds], lci[kCandLds];  // candidates stay in LDS when they fit
     const int unit = blockIdx.x;
     const int tid = threadIdx.x;
     if (tid == 0) {
@@ -249,35 +252,48 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
 
     const int lane = tid & 63;
     const unsigned long long lt = (1ull << lane) - 1ull;
-    for (uint32_t i0 = 0; i0 < n_s; i0 += kFinalThreads) {
-        const uint32_t i = i0 + tid;
-        uint32_t key = 0, bucket = 0xffffffffu, id = 0;
-        if (i < n_s) {
-            const uint2 p = su[i];
-            id = p.x;
-            dc_key_bucket(__uint_as_float(p.y), mode, key, bucket);
+    constexpr int kBatch = 4;  // survivor loads in flight per thread
+    for (uint32_t i0 = 0; i0 < n_s; i0 += kBatch * kFinalThreads) {
+        uint2 p[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const uint32_t i = i0 + j * kFinalThreads + tid;
+            p[j] = make_uint2(0u, 0u);
+            if (i < n_s) p[j] = su[i];
         }
-        // one LDS atomic per wave and list
-        const bool is_win = bucket < tb, is_cand = bucket == tb;
-        const unsigned long long mw = __ballot(is_win), mc = __ballot(is_cand);
-        if (mw) {
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(&s_win, (uint32_t)__popcll(mw));
-            base = __shfl(base, 0, 64);
-            const uint32_t slot = base + __popcll(mw & lt);
-            if (is_win && slot < kk) {
-                io[slot] = id;
-                if (ko) ko[slot] = key;
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const uint32_t i = i0 + j * kFinalThreads + tid;
+            uint32_t key = 0, bucket = 0xffffffffu;
+            const uint32_t id = p[j].x;
+            if (i < n_s) dc_key_bucket(__uint_as_float(p[j].y), mode, key, bucket);
+            // one LDS atomic per wave and list
+            const bool is_win = bucket < tb, is_cand = bucket == tb;
+            const unsigned long long mw = __ballot(is_win), mc = __ballot(is_cand);
+            if (mw) {
+                uint32_t base = 0;
+                if (lane == 0) base = atomicAdd(&s_win, (uint32_t)__popcll(mw));
+                base = __shfl(base, 0, 64);
+                const uint32_t slot = base + __popcll(mw & lt);
+                if (is_win && slot < kk) {
+                    io[slot] = id;
+                    if (ko) ko[slot] = key;
+                }
             }
-        }
-        if (mc) {
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(&s_cand, (uint32_t)__popcll(mc));
-            base = __shfl(base, 0, 64);
-            const uint32_t slot = base + __popcll(mc & lt);
-            if (is_cand && slot < (uint32_t)n_rows) {
-                ck[slot] = key;
-                ci[slot] = id;
+            if (mc) {
+                uint32_t base = 0;
+                if (lane == 0) base = atomicAdd(&s_cand, (uint32_t)__popcll(mc));
+                base = __shfl(base, 0, 64);
+                const uint32_t slot = base + __popcll(mc & lt);
+                if (is_cand) {
+                    if (slot < (uint32_t)kCandLds) {
+                        lck[slot] = key;
+                        lci[slot] = id;
+                    } else if (slot < (uint32_t)n_rows) {
+                        ck[slot] = key;
+                        ci[slot] = id;
+                    }
+                }
             }
         }
     }
@@ -297,7 +313,17 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
     if (c_less >= kk) return;
     uint32_t need = kk - c_less;
     if (need > n_c) need = n_c;
-    dc_finalize_unit(ck, ci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc,
+    const uint32_t *fk = lck, *fi = lci;
+    if (n_c > (uint32_t)kCandLds) {  // overflow: the head of the list joins the tail in global memory
+        for (int i = tid; i < kCandLds; i += kFinalThreads) {
+            ck[i] = lck[i];
+            ci[i] = lci[i];
+        }
+        __syncthreads();
+        fk = ck;
+        fi = ci;
+    }
+    dc_finalize_unit(fk, fi, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc,
                      ko ? ko + c_less : nullptr);
 }
 
@@ -349,7 +375,7 @@ extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k
 namespace {
 
 struct FusedPlan {
-    int n_units, k_eff, small_chunks;
+    int n_units, k_eff, small_chunks, big_steps;
     int64_t blocks;
 };
 
@@ -361,9 +387,11 @@ int plan_fused(const char *who, int n_b, int n_h, int n_rows, int budget, FusedP
     p->k_eff = budget < n_rows ? budget : n_rows;
     // chunks per unit: up to kSmallChunks blocks of 256 rows, then blocks of 2048 rows
     const int64_t tiles = ((int64_t)n_rows + kRowsPerBlockStep - 1) / kRowsPerBlockStep;
+    p->big_steps = kBigSteps;
     p->small_chunks = (int)(tiles < kSmallChunks ? tiles : kSmallChunks);
     const int64_t rest = (int64_t)n_rows - (int64_t)p->small_chunks * kRowsPerBlockStep;
-    const int64_t big_chunks = rest > 0 ? (rest + kStage - 1) / kStage : 0;
+    const int64_t big_rows = (int64_t)p->big_steps * kRowsPerBlockStep;
+    const int64_t big_chunks = rest > 0 ? (rest + big_rows - 1) / big_rows : 0;
     p->blocks = n_units64 * (p->small_chunks + big_chunks);
     DC_REQUIRE(p->blocks < (1ll << 31), "%s: grid too large", who);
     return DC_OK;
@@ -418,7 +446,8 @@ extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_
 #define DC_LAUNCH_SP(HD)                                                                           \
     hipLaunchKernelGGL(score_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st,    \
                        (const uint16_t *)k, (const uint16_t *)q, w.hist, w.state, w.surv,          \
-                       p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode, p.k_eff, p.small_chunks)
+                       p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode, p.k_eff, p.small_chunks,  \
+                       p.big_steps)
     if (hd == 64) DC_LAUNCH_SP(64);
     else if (hd == 128) DC_LAUNCH_SP(128);
     else DC_LAUNCH_SP(256);
