@@ -131,9 +131,11 @@ def alloc_workspace(nbytes: int, device) -> torch.Tensor:
 # wrappers
 # ---------------------------------------------------------------------------
 
-def group_mean(q: torch.Tensor, group: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """q (..., group, hd) bf16 viewed as (n_units, group, hd) -> (n_units, hd) bf16."""
-    hd = q.shape[-1]
+def group_mean(q: torch.Tensor, group: int, out: Optional[torch.Tensor] = None,
+               hd: Optional[int] = None) -> torch.Tensor:
+    """q bf16 holding (n_units, group, hd) values in that order -> (n_units, hd) bf16.
+    ``hd`` defaults to the last dimension of q."""
+    hd = q.shape[-1] if hd is None else hd
     q = q.contiguous()
     n_units = q.numel() // (group * hd)
     if out is None:

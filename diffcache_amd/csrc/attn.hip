@@ -299,10 +299,18 @@ int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const u
 
 }  // namespace
 
+// Upper bound of plan_attn(n_units, n).n_splits over every n <= n_total, so that a
+// workspace sized for the longest attended list also serves shorter ones.
+static int max_splits(int n_units, int n_total) {
+    int want = (1024 + n_units - 1) / (n_units > 0 ? n_units : 1);
+    int by_cap = (n_total + kMaxRowsPerSplit - 1) / kMaxRowsPerSplit;
+    int m = want > by_cap ? want : by_cap;
+    return m < 1 ? 1 : m;
+}
+
 extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attended) {
     if (n_units <= 0 || group <= 0 || hd <= 0) return 256;
-    AttnPlan p = plan_attn(n_units, n_rows_attended);
-    size_t slots = (size_t)n_units * p.n_splits;
+    size_t slots = (size_t)n_units * max_splits(n_units, n_rows_attended);
     return dc_align_up(slots * group * hd * 4, 256) + dc_align_up(slots * group * 2 * 4, 256);
 }
 
@@ -333,15 +341,15 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
     const int n_units = n_b * n_h;
     if (n_units == 0) return DC_OK;
     const int n_total = n_idx + n_sink + n_recent + (new_k ? 1 : 0);
-    const size_t need = dc_attn_workspace_bytes(n_units, group, hd, n_total);
+    AttnPlan plan = plan_attn(n_units, n_total);
+    const size_t slots = (size_t)n_units * plan.n_splits;
+    const size_t need = dc_align_up(slots * group * hd * 4, 256) + dc_align_up(slots * group * 2 * 4, 256);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "dc_gather_attn_bf16: workspace must be non-null and 256-byte aligned");
     if (workspace_bytes < need) {
         dc_set_error("dc_gather_attn_bf16: workspace %zu bytes < %zu needed", workspace_bytes, need);
         return DC_ENOMEM;
     }
-    AttnPlan plan = plan_attn(n_units, n_total);
-    const size_t slots = (size_t)n_units * plan.n_splits;
     float *ws_acc = (float *)workspace;
     float *ws_ml = (float *)((char *)workspace + dc_align_up(slots * group * hd * 4, 256));
     hipStream_t st = (hipStream_t)stream;

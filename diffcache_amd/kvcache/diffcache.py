@@ -1,0 +1,303 @@
+"""``DiffCache``: the reference's KV-cache operator API on an HBM-resident store.
+
+Constructor and method names, argument meaning and call order are those of
+``src/diffcache/kvcache/diffcache.py:15-300`` so the model harness
+(``src/diffcache/base.py:83,125,133,151-154,174,210,242``) can use it unchanged:
+
+    prefill_update_kv_cache(key_states, value_states, layer_idx)
+    get_kvcache(layer_idx)
+    decode_pre_query_operation(queries)      # inside the captured pre-attention graph
+    decode_query_kvcache(layer_idx)          # between the two graphs
+    decode_post_query_operation(layer_idx)   # inside the captured post-attention graph
+    seq_len / seq_len_gpu, save_prefill_cache / load_prefill_cache
+
+What changed underneath.  The reference keeps only ``budget + prefix +
+suffix_max`` rows per head on the GPU and sends every decode query through the
+host (D2H, device sync, Rust search, H2D).  Here all K/V rows of every layer
+stay in HBM as bf16 ``(bsz, kv_heads, max_length, head_dim)``; the three hooks
+enqueue the group-mean, the exact scan + top-k, and a device-side row gather on
+the current stream, with no host synchronisation and no allocation, so they
+are capturable.  ``kbuf`` / ``vbuf`` keep the reference's geometry
+``[retrieved (right aligned) | prefix | suffix]`` for harnesses that run their
+own attention over ``get_kvcache()``.
+
+``decode_attention`` is the native path that has no counterpart in the
+reference: score -> select -> attention straight from the store (one C call),
+replacing the ``flash_attn_with_kvcache`` call of ``base.py:134-142`` as well.
+"""
+from __future__ import annotations
+
+import json
+import os
+from typing import List, Optional
+
+import torch
+
+from .. import _hip as hip
+from ..data_layer import DiffCacheHIP, init_metrics
+
+
+class DiffCache:
+    def __init__(
+        self,
+        num_layers: int,
+        batch_size: int,
+        max_length: int,
+        num_kv_heads: int,
+        num_q_heads: int,
+        head_dim: int,
+        retrieval_budget: int,
+        nsw_m: int,
+        nsw_ef_cons: int,
+        kvbuf_prefix_len: int,
+        kvbuf_suffix_len: int,
+        kvbuf_suffix_maxlen: int,
+        attn_mass_threshold: float,
+        k_check_seq: List[int],
+        r_sq: List[List[float]],
+        key_mode: str = "ref_dist",
+        device: str = "cuda",
+    ) -> None:
+        self.num_layers = num_layers
+        self.batch_size = batch_size
+        self.max_length = max_length
+        self.num_kv_heads = num_kv_heads
+        self.num_q_heads = num_q_heads
+        self.head_dim = head_dim
+        self.retrieval_budget = retrieval_budget
+        self.nsw_m = nsw_m
+        self.nsw_ef_cons = nsw_ef_cons
+        self.r_sq = r_sq
+        self.attn_mass_threshold = attn_mass_threshold
+        self.k_check_seq = k_check_seq
+        self.key_mode = key_mode
+        self.mode = hip.MODE_REF_DIST if key_mode == "ref_dist" else hip.MODE_IP
+        self.device = torch.device(device)
+        self.data_layers: List[Optional[DiffCacheHIP]] = [None for _ in range(num_layers)]
+        self.retrieval_region_len = 0
+
+        # kvbuf geometry of the reference (diffcache.py:48-66):
+        #   [ retrieval_budget | prefix_len | suffix_maxlen ], layout (bsz, kh, seq, hd)
+        self.kvbuf_suffix_maxlen = kvbuf_suffix_maxlen
+        self.kvbuf_prefix_len = kvbuf_prefix_len
+        self.kvbuf_suffix_len = kvbuf_suffix_len
+        kvbuf_len = retrieval_budget + kvbuf_prefix_len + kvbuf_suffix_maxlen
+        shape = (batch_size, num_kv_heads, kvbuf_len, head_dim)
+        self.kbuf = [torch.empty(shape, device=self.device, dtype=torch.bfloat16) for _ in range(num_layers)]
+        self.vbuf = [torch.empty(shape, device=self.device, dtype=torch.bfloat16) for _ in range(num_layers)]
+
+        # the HBM-resident store that replaces the host index: every row of every layer
+        store = (batch_size, num_kv_heads, max_length, head_dim)
+        self.kstore = [torch.zeros(store, device=self.device, dtype=torch.bfloat16) for _ in range(num_layers)]
+        self.vstore = [torch.zeros(store, device=self.device, dtype=torch.bfloat16) for _ in range(num_layers)]
+
+        n_units = batch_size * num_kv_heads
+        self.group = num_q_heads // num_kv_heads
+        # group-mean query of the current layer (the reference's pinned qbuf_cpu, diffcache.py:80)
+        self.qbuf = torch.zeros((batch_size, num_kv_heads, head_dim), device=self.device, dtype=torch.bfloat16)
+        # selected node ids of every layer, relative to the retrieval region, best first
+        self.idx = [torch.zeros((n_units, max(retrieval_budget, 1)), device=self.device, dtype=torch.int32)
+                    for _ in range(num_layers)]
+        self._ws: Optional[torch.Tensor] = None
+        self._ws_rows = -1
+        self._attn_out: Optional[torch.Tensor] = None
+        self._prefix0 = kvbuf_prefix_len
+        self._suffix0 = kvbuf_suffix_len
+
+        init_metrics()
+
+    # ------------------------------------------------------------------ helpers
+    def _region(self):
+        lo = self.kvbuf_prefix_len
+        return lo, lo + self.retrieval_region_len
+
+    def _ensure_workspace(self) -> torch.Tensor:
+        region = self.retrieval_region_len
+        if self._ws is None or self._ws_rows != region:
+            n_units = self.batch_size * self.num_kv_heads
+            attended = min(region, self.retrieval_budget) + self.kvbuf_prefix_len + self.kvbuf_suffix_maxlen + 1
+            self._ws = hip.alloc_workspace(
+                hip.layer_workspace_bytes(n_units, region, self.retrieval_budget, self.group,
+                                          self.head_dim, attended), self.device)
+            self._ws_rows = region
+        return self._ws
+
+    # ------------------------------------------------------------------ prefill
+    def prefill_update_kv_cache(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int):
+        """key_states / value_states (bsz, seq_len, num_kv_heads, head_dim) bf16 on the
+        GPU (diffcache.py:149-184)."""
+        seq_len = key_states.size(1)
+        assert seq_len <= self.max_length, "prompt longer than max_length"
+
+        # r_sq from the prefill keys, as the reference does; only the graph build needed it
+        r_sq = torch.einsum("bshd,bshd->bsh", key_states, key_states).max(dim=1).values.max(dim=0).values.tolist()
+        self.r_sq[layer_idx] = r_sq
+
+        # all rows into the store, (b, s, h, d) -> (b, h, s, d)
+        hip.ingest_kv(self.kstore[layer_idx], key_states, 0)
+        hip.ingest_kv(self.vstore[layer_idx], value_states, 0)
+
+        prefix_len = min(self._prefix0, seq_len)                    # diffcache.py:163
+        suffix_len = min(self._suffix0, seq_len - prefix_len)       # diffcache.py:169
+        self.kvbuf_prefix_len = prefix_len
+        self.kvbuf_suffix_len = suffix_len
+        self.retrieval_region_len = seq_len - prefix_len - suffix_len
+
+        # prefix and suffix rows of the assembled buffer (diffcache.py:164-171)
+        b0 = self.retrieval_budget
+        ks, vs = self.kstore[layer_idx], self.vstore[layer_idx]
+        self.kbuf[layer_idx][:, :, b0:b0 + prefix_len].copy_(ks[:, :, :prefix_len])
+        self.vbuf[layer_idx][:, :, b0:b0 + prefix_len].copy_(vs[:, :, :prefix_len])
+        s0 = seq_len - suffix_len
+        self.kbuf[layer_idx][:, :, b0 + prefix_len:b0 + prefix_len + suffix_len].copy_(ks[:, :, s0:seq_len])
+        self.vbuf[layer_idx][:, :, b0 + prefix_len:b0 + prefix_len + suffix_len].copy_(vs[:, :, s0:seq_len])
+
+        self._bind_data_layer(layer_idx)
+        return key_states, value_states
+
+    def _bind_data_layer(self, layer_idx: int) -> None:
+        """The layer's retrieval region seen through the reference's data-layer API."""
+        lo, hi = self._region()
+        n = hi - lo
+        self.data_layers[layer_idx] = DiffCacheHIP(
+            bsz=self.batch_size, q_head_num=self.num_q_heads, kv_head_num=self.num_kv_heads,
+            head_dim=self.head_dim, max_ctx_len=n, m=self.nsw_m, ef_cons=self.nsw_ef_cons,
+            r_sq=self.r_sq[layer_idx], name=f"l{layer_idx:03d}",
+            attn_mass_threshold=self.attn_mass_threshold, k_check_seq=self.k_check_seq,
+            key_mode=self.key_mode, device=str(self.device),
+            storage=(self.kstore[layer_idx][:, :, lo:hi], self.vstore[layer_idx][:, :, lo:hi]))
+        self.data_layers[layer_idx].ctx_len = n
+
+    def get_kvcache(self, layer_idx: int):
+        retrieval_len = min(self.retrieval_region_len, self.retrieval_budget)
+        start = self.retrieval_budget - retrieval_len
+        return (self.kbuf[layer_idx][:, :, start:, :].permute(0, 2, 1, 3),
+                self.vbuf[layer_idx][:, :, start:, :].permute(0, 2, 1, 3))
+
+    # ------------------------------------------------------------------ decode hooks
+    def decode_pre_query_operation(self, queries: torch.Tensor) -> None:
+        """GQA-group mean of the layer's queries (diffcache.py:191-194), kept on the device."""
+        hip.group_mean(queries, self.group, out=self.qbuf.view(-1, self.head_dim), hd=self.head_dim)
+
+    def decode_query_kvcache(self, layer_idx: int) -> None:
+        """Exact scan + top-k of the retrieval region with the mean query
+        (diffcache.py:211-223 -> lib.rs:373-404 -> nsw.rs:592-630)."""
+        retrieval_len = min(self.retrieval_region_len, self.retrieval_budget)
+        if retrieval_len > 0:
+            lo, hi = self._region()
+            ws = self._ensure_workspace()
+            hip.score_select(self.kstore[layer_idx], self.qbuf, lo, hi - lo, retrieval_len, self.mode,
+                             hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
+        assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
+        if layer_idx == self.num_layers - 1:
+            self.kvbuf_suffix_len += 1
+
+    def decode_post_query_operation(self, layer_idx: int) -> None:
+        """Selected rows into kbuf/vbuf[:, :, budget - len : budget] (diffcache.py:196-209)."""
+        retrieval_len = min(self.retrieval_region_len, self.retrieval_budget)
+        if retrieval_len <= 0:
+            return
+        lo, _ = self._region()
+        b0 = self.retrieval_budget
+        hip.gather_rows(self.kstore[layer_idx], self.vstore[layer_idx], self.idx[layer_idx],
+                        self.kbuf[layer_idx][:, :, b0 - retrieval_len:b0],
+                        self.vbuf[layer_idx][:, :, b0 - retrieval_len:b0], row_offset=lo, n_idx=retrieval_len)
+
+    # ------------------------------------------------------------------ native decode path
+    def decode_attention(self, layer_idx: int, queries: torch.Tensor, key_states: torch.Tensor,
+                         value_states: torch.Tensor, out: Optional[torch.Tensor] = None,
+                         order: int = hip.ORDER_ANY) -> torch.Tensor:
+        """One layer of the decode path in one call: append the token's k/v to the
+        store, score the retrieval region with the group-mean query, select the
+        exact top-``retrieval_budget``, attend over [selected | prefix | suffix +
+        this token].  queries (bsz, 1, Hq*hd) or (bsz, Hq, hd); key/value_states
+        (bsz, 1, Hkv, hd).  Returns (bsz, Hq, hd) bf16.  Call it for every layer of
+        a step; the suffix grows by one after the last layer."""
+        b, hq, hkv, hd = self.batch_size, self.num_q_heads, self.num_kv_heads, self.head_dim
+        assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
+        lo, hi = self._region()
+        pos = hi + self.kvbuf_suffix_len
+        assert pos < self.max_length, "store is full"
+        q = queries.reshape(b, hq, hd)
+        if not q.is_contiguous():
+            q = q.contiguous()
+        hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], key_states.reshape(b, hkv, hd),
+                      value_states.reshape(b, hkv, hd), pos)
+        if out is None:
+            if self._attn_out is None:
+                self._attn_out = torch.empty((b, hq, hd), device=self.device, dtype=torch.bfloat16)
+            out = self._attn_out
+        ws = self._ensure_workspace()
+        hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
+                         self.kvbuf_suffix_len + 1, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
+                         mode=self.mode, order=order)
+        if layer_idx == self.num_layers - 1:
+            self.kvbuf_suffix_len += 1
+        return out
+
+    # ------------------------------------------------------------------ prefill cache
+    def save_prefill_cache(self, prefill_cache_path: str) -> None:
+        """Same directory layout as diffcache.py:225-259."""
+        path = os.path.join(prefill_cache_path, "metadata.txt")
+        metadata = {
+            "r_sq": self.r_sq,
+            "kvbuf_prefix_len": self.kvbuf_prefix_len,
+            "kvbuf_suffix_len": self.kvbuf_suffix_len,
+            "retrieval_region_len": self.retrieval_region_len,
+        }
+        with open(path, "w") as f:
+            json.dump(metadata, f)
+        b0, p, s = self.retrieval_budget, self.kvbuf_prefix_len, self.kvbuf_suffix_len
+        for layer_idx in range(self.num_layers):
+            layer_path = os.path.join(prefill_cache_path, f"p_l_{layer_idx:03d}")
+            os.makedirs(layer_path, exist_ok=False)
+            torch.save(self.kbuf[layer_idx][:, :, b0:b0 + p, :], os.path.join(layer_path, "k.pt"))
+            torch.save(self.vbuf[layer_idx][:, :, b0:b0 + p, :], os.path.join(layer_path, "v.pt"))
+        for layer_idx in range(self.num_layers):
+            layer_path = os.path.join(prefill_cache_path, f"s_l_{layer_idx:03d}")
+            os.makedirs(layer_path, exist_ok=False)
+            torch.save(self.kbuf[layer_idx][:, :, b0 + p:b0 + p + s, :], os.path.join(layer_path, "k.pt"))
+            torch.save(self.vbuf[layer_idx][:, :, b0 + p:b0 + p + s, :], os.path.join(layer_path, "v.pt"))
+        for layer_idx in range(self.num_layers):
+            layer_path = os.path.join(prefill_cache_path, f"d_l_{layer_idx:03d}")
+            os.makedirs(layer_path, exist_ok=False)
+            self.data_layers[layer_idx].save(layer_path)
+
+    def load_prefill_cache(self, inputs_ids: torch.Tensor, prefill_cache_path: str) -> None:
+        """diffcache.py:261-293; the K/V rows come back into the HBM store."""
+        ctx_len = inputs_ids.size(1)
+        with open(os.path.join(prefill_cache_path, "metadata.txt"), "r") as f:
+            metadata = json.load(f)
+        self.r_sq = metadata["r_sq"]
+        self.kvbuf_prefix_len = metadata["kvbuf_prefix_len"]
+        self.kvbuf_suffix_len = metadata["kvbuf_suffix_len"]
+        self.retrieval_region_len = metadata["retrieval_region_len"]
+        b0, p, s = self.retrieval_budget, self.kvbuf_prefix_len, self.kvbuf_suffix_len
+        lo, hi = self._region()
+        for layer_idx in range(self.num_layers):
+            pp = os.path.join(prefill_cache_path, f"p_l_{layer_idx:03d}")
+            sp = os.path.join(prefill_cache_path, f"s_l_{layer_idx:03d}")
+            pk = torch.load(os.path.join(pp, "k.pt"), weights_only=True).to(self.device)
+            pv = torch.load(os.path.join(pp, "v.pt"), weights_only=True).to(self.device)
+            sk = torch.load(os.path.join(sp, "k.pt"), weights_only=True).to(self.device)
+            sv = torch.load(os.path.join(sp, "v.pt"), weights_only=True).to(self.device)
+            self.kbuf[layer_idx][:, :, b0:b0 + p, :] = pk
+            self.vbuf[layer_idx][:, :, b0:b0 + p, :] = pv
+            self.kbuf[layer_idx][:, :, b0 + p:b0 + p + s, :] = sk
+            self.vbuf[layer_idx][:, :, b0 + p:b0 + p + s, :] = sv
+            self.kstore[layer_idx][:, :, :p] = pk
+            self.vstore[layer_idx][:, :, :p] = pv
+            self.kstore[layer_idx][:, :, hi:hi + s] = sk
+            self.vstore[layer_idx][:, :, hi:hi + s] = sv
+        for layer_idx in range(self.num_layers):
+            self._bind_data_layer(layer_idx)
+            layer_path = os.path.join(prefill_cache_path, f"d_l_{layer_idx:03d}")
+            self.data_layers[layer_idx].load(layer_path, ctx_len)
+            self.data_layers[layer_idx].update_r_sq(self.r_sq[layer_idx])
+
+    def seq_len(self, layer_idx: int) -> int:
+        return self.kvbuf_prefix_len + self.kvbuf_suffix_len + self.retrieval_region_len
+
+    def seq_len_gpu(self, layer_idx: int) -> int:
+        retrieval_len = min(self.retrieval_region_len, self.retrieval_budget)
+        return self.kvbuf_prefix_len + self.kvbuf_suffix_len + retrieval_len

@@ -1,0 +1,292 @@
+"""GPU parity of the two host classes that mirror the reference's interfaces:
+``DiffCacheHIP`` (lib.rs ``DiffCacheCPU``) against the C restatement of the
+exact scan, and ``DiffCache`` (kvcache/diffcache.py) against the numpy oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_ref
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rand_bf16(rng, *shape, scale=1.0):
+    return orc.f32_to_bf16((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+def dev_bf16(u16):
+    return torch.from_numpy(u16.view(np.int16).copy()).view(torch.bfloat16).to(DEV)
+
+
+def np_u16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def bf16_close(got_f32, want_f64):
+    tol = np.maximum(2e-3, np.abs(want_f64) * 2.0 ** -8)
+    return bool(np.all(np.abs(got_f32 - want_f64) <= tol))
+
+
+# ---------------------------------------------------------------- DiffCacheHIP
+
+def test_data_layer_query_equals_cpu_reference_rows():
+    """prefill + query with numpy u16 in/out, the calling convention of
+    diffcache.py:147,218-220; integer-valued data makes every fp32 accumulation
+    order exact, so rows must match the C restatement of nsw.rs:592-630 bit for bit."""
+    from diffcache_amd import DiffCacheHIP, init_metrics, metrics
+    init_metrics()
+    rng = np.random.default_rng(1)
+    b, hq, hkv, hd, n, ef = 2, 8, 2, 128, 3000, 256
+    keys = orc.f32_to_bf16(rng.integers(-3, 4, (b, hkv, n, hd)).astype(np.float32))
+    vals = rand_bf16(rng, b, hkv, n, hd)
+    q = orc.f32_to_bf16(rng.integers(-2, 3, (b, hkv, hd)).astype(np.float32))
+    dl = DiffCacheHIP(b, hq, hkv, hd, max_ctx_len=4096, name="l007", use_bruteforce=True)
+    neighbours = np.zeros((b, hkv, n, 32), np.uint32)
+    dl.prefill(keys, vals, neighbours)
+    out_k = np.zeros((b, hkv, ef, hd), np.uint16)
+    out_v = np.zeros((b, hkv, ef, hd), np.uint16)
+    dl.query(out_k, out_v, q, ef)
+    ck, cv, cids = cpu_ref.query(keys, vals, q, ef, n_threads=4)
+    assert np.array_equal(out_k, ck) and np.array_equal(out_v, cv)
+    ids = dl.query_ids(q, ef).cpu().numpy().astype(np.uint32).reshape(b, hkv, ef)
+    assert np.array_equal(ids, cids)
+    m = metrics()
+    assert m["l007_num_searches"] == b * hkv and m["l007_total_query_latency"] > 0
+    # keys come back as f32 (lib.rs:646-649)
+    assert np.array_equal(dl.get_keys(), orc.bf16_to_f32(keys))
+
+
+def test_data_layer_random_data_ids_follow_gpu_scores():
+    from diffcache_amd import DiffCacheHIP
+    rng = np.random.default_rng(2)
+    b, hq, hkv, hd, n, ef = 1, 4, 4, 128, 20000, 1024
+    keys, vals = rand_bf16(rng, b, hkv, n, hd), rand_bf16(rng, b, hkv, n, hd)
+    q = rand_bf16(rng, b, hkv, hd)
+    for key_mode, mode in (("ref_dist", orc.MODE_REF_DIST), ("ip", orc.MODE_IP)):
+        dl = DiffCacheHIP(b, hq, hkv, hd, max_ctx_len=n, key_mode=key_mode)
+        dl.prefill(dev_bf16(keys), dev_bf16(vals))
+        ids, scores = dl.query_ids(dev_bf16(q), ef, return_scores=True)
+        ids2 = dl.query_ids(dev_bf16(q), ef)                         # streaming path
+        sc = scores.cpu().numpy()
+        for u in range(hkv):
+            want = orc.topk_select(sc[u], ef, mode)
+            assert np.array_equal(ids.cpu().numpy()[u].astype(np.uint32), want)
+            assert np.array_equal(ids2.cpu().numpy()[u].astype(np.uint32), want)
+            ref = orc.scores_f64(q[0, u], keys[0, u])
+            assert np.max(np.abs(sc[u] - ref)) <= 1e-5 * np.max(np.abs(ref)) + 1e-4
+
+
+def test_data_layer_insert_ef_clamp_and_device_outputs():
+    from diffcache_amd import DiffCacheHIP
+    rng = np.random.default_rng(3)
+    b, hkv, hd = 1, 2, 64
+    dl = DiffCacheHIP(b, 4, hkv, hd, max_ctx_len=64)
+    keys = orc.f32_to_bf16(rng.integers(-3, 4, (b, hkv, 10, hd)).astype(np.float32))
+    vals = rand_bf16(rng, b, hkv, 10, hd)
+    dl.prefill(keys, vals)
+    extra_k = orc.f32_to_bf16(rng.integers(-3, 4, (5, b, hkv, hd)).astype(np.float32))
+    extra_v = rand_bf16(rng, 5, b, hkv, hd)
+    for i in range(5):
+        dl.insert(extra_k[i], extra_v[i])
+    assert dl.ctx_len == 15
+    all_k = np.concatenate([keys, np.transpose(extra_k, (1, 2, 0, 3))], axis=2)
+    all_v = np.concatenate([vals, np.transpose(extra_v, (1, 2, 0, 3))], axis=2)
+    q = orc.f32_to_bf16(rng.integers(-2, 3, (b, hkv, hd)).astype(np.float32))
+    out_k = torch.zeros((b, hkv, 40, hd), dtype=torch.bfloat16, device=DEV)
+    out_v = torch.zeros_like(out_k)
+    dl.query(out_k, out_v, q, 40)                       # ef 40 > ctx 15 -> 15 rows (lib.rs:374)
+    ck, cv, _ = cpu_ref.query(all_k, all_v, q, 40)
+    assert ck.shape[2] == 15
+    assert np.array_equal(np_u16(out_k)[:, :, :15], ck) and np.array_equal(np_u16(out_v)[:, :, :15], cv)
+    assert np.all(np_u16(out_k)[:, :, 15:] == 0)
+    # raw-pointer variant (lib.rs:626-636)
+    sk = torch.zeros((b, hkv, 15, hd), dtype=torch.bfloat16, device=DEV)
+    sv = torch.zeros_like(sk)
+    dl.query_streaming(torch.cuda.current_stream().cuda_stream, sk.data_ptr(), sv.data_ptr(), q, 15)
+    torch.cuda.synchronize()
+    assert np.array_equal(np_u16(sk), ck) and np.array_equal(np_u16(sv), cv)
+    with pytest.raises(AssertionError):
+        dl.update_r_sq([1.0])                           # lib.rs:652
+    with pytest.raises(AssertionError):
+        dl.query(out_k, out_v, np.zeros((b, hkv + 1, hd), np.uint16), 4)
+
+
+def test_data_layer_save_load_roundtrip(tmp_path):
+    from diffcache_amd import DiffCacheHIP
+    rng = np.random.default_rng(4)
+    b, hkv, hd, n = 1, 2, 64, 500
+    keys, vals = rand_bf16(rng, b, hkv, n, hd), rand_bf16(rng, b, hkv, n, hd)
+    dl = DiffCacheHIP(b, 2, hkv, hd, max_ctx_len=512, r_sq=[2.5, 3.5])
+    dl.prefill(keys, vals)
+    prefix = str(tmp_path / "d_l_000")                  # files land beside it: d_l_000b000_h000.idx
+    dl.save(prefix)
+    assert os.path.exists(prefix + "b000_h001.idx")
+    dl2 = DiffCacheHIP(b, 2, hkv, hd, max_ctx_len=512)
+    dl2.load(prefix, 100000)                            # the reference passes the full prompt length
+    assert dl2.ctx_len == n and dl2.r_sq == [2.5, 3.5]
+    assert np.array_equal(np_u16(dl2.keys[:, :, :n]), keys) and np.array_equal(np_u16(dl2.vals[:, :, :n]), vals)
+
+
+# ---------------------------------------------------------------- DiffCache
+
+def make_cache(num_layers, b, max_len, hkv, hq, hd, budget, p, s, smax, key_mode="ref_dist"):
+    from diffcache_amd import DiffCache
+    return DiffCache(num_layers=num_layers, batch_size=b, max_length=max_len, num_kv_heads=hkv,
+                     num_q_heads=hq, head_dim=hd, retrieval_budget=budget, nsw_m=16, nsw_ef_cons=200,
+                     kvbuf_prefix_len=p, kvbuf_suffix_len=s, kvbuf_suffix_maxlen=smax,
+                     attn_mass_threshold=0.9, k_check_seq=[1048576],
+                     r_sq=[[4.0] * hkv for _ in range(num_layers)], key_mode=key_mode)
+
+
+@pytest.mark.parametrize("seq", [3000, 150])
+def test_diffcache_hooks_assemble_the_reference_buffer(seq):
+    """The reference call order (base.py:150-155) through the kept hooks; the
+    assembled kbuf/vbuf view must hold [retrieved best-first | prefix | suffix]."""
+    rng = np.random.default_rng(10 + seq)
+    L, b, hkv, hq, hd, budget, p, s, smax = 2, 2, 2, 8, 128, 256, 16, 32, 64
+    g = hq // hkv
+    cache = make_cache(L, b, seq + 40, hkv, hq, hd, budget, p, s, smax)
+    ks = [orc.f32_to_bf16(rng.integers(-3, 4, (b, seq, hkv, hd)).astype(np.float32)) for _ in range(L)]
+    vs = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    for l in range(L):
+        k_dev, v_dev = dev_bf16(ks[l]), dev_bf16(vs[l])
+        rk, rv = cache.prefill_update_kv_cache(k_dev, v_dev, l)
+        assert rk is k_dev and rv is v_dev
+    p_len, s_len, lo, hi = orc.region_split(seq, p, s)
+    assert (cache.kvbuf_prefix_len, cache.kvbuf_suffix_len, cache.retrieval_region_len) == (p_len, s_len, hi - lo)
+    assert cache.seq_len(0) == seq and cache.seq_len_gpu(0) == p_len + s_len + min(budget, hi - lo)
+    r_len = min(budget, hi - lo)
+    for l in range(L):
+        q = orc.f32_to_bf16((rng.integers(-2, 3, (b, 1, hq * hd))).astype(np.float32))
+        cache.decode_pre_query_operation(dev_bf16(q))
+        cache.decode_query_kvcache(l)
+        cache.decode_post_query_operation(l)
+        kc, vc = cache.get_kvcache(l)                       # (b, S, hkv, hd) views
+        assert kc.shape[1] == r_len + p_len + smax
+        kc, vc = np_u16(kc), np_u16(vc)
+        qmean = orc.group_mean_bf16(q.reshape(b, hq, hd), hkv)
+        assert np.array_equal(np_u16(cache.qbuf), qmean)
+        for bi in range(b):
+            for h in range(hkv):
+                K, V = ks[l][bi, :, h], vs[l][bi, :, h]
+                sel = orc.topk_select(orc.scores_f32(qmean[bi, h], K[lo:hi]), budget, orc.MODE_REF_DIST)
+                rows = orc.attended_rows(sel, p_len, hi, seq)
+                n_att = r_len + p_len + s_len
+                assert np.array_equal(kc[bi, :n_att, h], K[rows])
+                assert np.array_equal(vc[bi, :n_att, h], V[rows])
+    assert cache.kvbuf_suffix_len == s_len + 1               # grows once per step (diffcache.py:222-223)
+
+
+@pytest.mark.parametrize("key_mode", ["ref_dist", "ip"])
+def test_diffcache_decode_attention_matches_oracle_over_steps(key_mode):
+    rng = np.random.default_rng(20)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 2, 2, 2, 8, 128, 128, 4, 16, 32, 2000
+    mode = orc.MODE_REF_DIST if key_mode == "ref_dist" else orc.MODE_IP
+    cache = make_cache(L, b, seq + 64, hkv, hq, hd, budget, p, s, smax, key_mode)
+    K = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    V = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    for l in range(L):
+        cache.prefill_update_kv_cache(dev_bf16(K[l]), dev_bf16(V[l]), l)
+    hist_k = [np.transpose(K[l], (0, 2, 1, 3)).copy() for l in range(L)]      # (b, hkv, n, hd)
+    hist_v = [np.transpose(V[l], (0, 2, 1, 3)).copy() for l in range(L)]
+    p_len, s_len, lo, hi = orc.region_split(seq, p, s)
+    from diffcache_amd import _hip
+    for step in range(3):
+        for l in range(L):
+            q = rand_bf16(rng, b, 1, hq * hd)
+            nk, nv = rand_bf16(rng, b, 1, hkv, hd), rand_bf16(rng, b, 1, hkv, hd)
+            out = cache.decode_attention(l, dev_bf16(q), dev_bf16(nk), dev_bf16(nv), order=_hip.ORDER_BEST)
+            torch.cuda.synchronize()
+            got = orc.bf16_to_f32(np_u16(out))
+            ids = cache.idx[l].cpu().numpy().astype(np.uint32)
+            # dense scores of the same arithmetic decide which ids are expected
+            qmean = orc.group_mean_bf16(q.reshape(b, hq, hd), hkv)
+            sc = _hip.score(cache.kstore[l], dev_bf16(qmean), lo, hi - lo,
+                            _hip.MODE_REF_DIST if key_mode == "ref_dist" else _hip.MODE_IP).cpu().numpy()
+            for bi in range(b):
+                # history = prompt + tokens of earlier steps; the oracle's region split sees
+                # the same fixed region when told the suffix is s_len + step rows long
+                res = orc.decode_layer(q.reshape(b, hq, hd)[bi], hist_k[l][bi], hist_v[l][bi], hkv, budget,
+                                       p, s_len + step, mode, nk[bi, 0], nv[bi, 0],
+                                       scores_override=sc[bi * hkv:(bi + 1) * hkv])
+                for h in range(hkv):
+                    assert np.array_equal(ids[bi * hkv + h, :budget], res["sel"][h])
+                assert bf16_close(got[bi], res["out"])
+            # the token becomes part of the history (suffix) for later steps
+            hist_k[l] = np.concatenate([hist_k[l], np.transpose(nk, (0, 2, 1, 3))], axis=2)
+            hist_v[l] = np.concatenate([hist_v[l], np.transpose(nv, (0, 2, 1, 3))], axis=2)
+        assert cache.kvbuf_suffix_len == s_len + step + 1
+
+
+def test_diffcache_hooks_under_graph_capture():
+    """decode_pre/post are called inside captured graphs in the reference
+    (base.py:121-125,132-133): capture them, replay with fresh inputs between
+    eager work, compare every replay with the eager result."""
+    rng = np.random.default_rng(30)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 1, 1, 2, 8, 128, 64, 4, 8, 32, 1500
+    cache = make_cache(L, b, seq + 40, hkv, hq, hd, budget, p, s, smax)
+    K, V = rand_bf16(rng, b, seq, hkv, hd), rand_bf16(rng, b, seq, hkv, hd)
+    cache.prefill_update_kv_cache(dev_bf16(K), dev_bf16(V), 0)
+    q_static = torch.zeros((b, 1, hq * hd), dtype=torch.bfloat16, device=DEV)
+    # warm up on a side stream as torch requires before capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        cache.decode_pre_query_operation(q_static)
+        cache.decode_query_kvcache(0)
+        cache.decode_post_query_operation(0)
+    torch.cuda.current_stream().wait_stream(side)
+    cache.kvbuf_suffix_len -= 1
+    g_pre, g_post = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_pre):
+        cache.decode_pre_query_operation(q_static)
+    with torch.cuda.graph(g_post):
+        cache.decode_post_query_operation(0)
+    for it in range(3):
+        q = rand_bf16(rng, b, 1, hq * hd)
+        q_static.copy_(dev_bf16(q))
+        g_pre.replay()
+        cache.decode_query_kvcache(0)
+        g_post.replay()
+        torch.cuda.synchronize()
+        kc_graph = np_u16(cache.get_kvcache(0)[0]).copy()
+        cache.kvbuf_suffix_len -= 1
+        cache.decode_pre_query_operation(q_static)
+        cache.decode_query_kvcache(0)
+        cache.decode_post_query_operation(0)
+        torch.cuda.synchronize()
+        cache.kvbuf_suffix_len -= 1
+        assert np.array_equal(kc_graph, np_u16(cache.get_kvcache(0)[0]))
+        (torch.randn(1000, device=DEV) * 2).sum().item()    # unrelated eager work between replays
+
+
+def test_diffcache_prefill_cache_roundtrip(tmp_path):
+    rng = np.random.default_rng(40)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 2, 1, 2, 4, 64, 32, 4, 8, 16, 300
+    cache = make_cache(L, b, seq + 20, hkv, hq, hd, budget, p, s, smax)
+    K = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    V = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    for l in range(L):
+        cache.prefill_update_kv_cache(dev_bf16(K[l]), dev_bf16(V[l]), l)
+    d = str(tmp_path / "c0")
+    os.makedirs(d)
+    cache.save_prefill_cache(d)
+    for name in ("metadata.txt", "p_l_000/k.pt", "s_l_001/v.pt", "d_l_000b000_h001.idx"):
+        assert os.path.exists(os.path.join(d, name)), name
+    cache2 = make_cache(L, b, seq + 20, hkv, hq, hd, budget, p, s, smax)
+    cache2.load_prefill_cache(torch.zeros((b, seq), dtype=torch.long), d)
+    assert cache2.retrieval_region_len == cache.retrieval_region_len
+    q = rand_bf16(rng, b, 1, hq * hd)
+    outs = []
+    for c in (cache, cache2):
+        c.decode_pre_query_operation(dev_bf16(q))
+        c.decode_query_kvcache(1)
+        c.decode_post_query_operation(1)
+        torch.cuda.synchronize()
+        n_att = c.seq_len_gpu(1) - 0
+        outs.append(np_u16(c.get_kvcache(1)[0])[:, :budget + p + s])
+    assert np.array_equal(outs[0], outs[1])

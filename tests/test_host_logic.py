@@ -1,0 +1,149 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header
+declares, the snapshot codec, option handling and refusal of CPU tensors.  No
+kernel is launched here."""
+import ctypes
+import json
+import os
+import re
+import struct
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from diffcache_amd import _hip
+    header = open(os.path.join(ROOT, "include", "diffcache_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(dc_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 20
+    lib = ctypes.CDLL(_hip.LIB_PATH)
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert declared == set(_hip.SYMBOLS), declared ^ set(_hip.SYMBOLS)
+    assert _hip.lib.dc_version() == 1
+
+
+def test_layer_args_struct_matches_header_order():
+    from diffcache_amd import _hip
+    header = open(os.path.join(ROOT, "include", "diffcache_hip.h")).read()
+    body = header[header.index("typedef struct dc_layer_args {"):header.index("} dc_layer_args;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.replace("typedef struct dc_layer_args {", "").strip()
+        if not decl:
+            continue
+        for part in decl.split(","):
+            names.append(re.findall(r"([A-Za-z_][A-Za-z0-9_]*)\s*$", part.strip())[0])
+    assert names == [f[0] for f in _hip.LayerArgs._fields_]
+
+
+def test_wrappers_refuse_cpu_tensors():
+    from diffcache_amd import _hip
+    k = torch.zeros((1, 1, 16, 128), dtype=torch.bfloat16)
+    q = torch.zeros((1, 1, 128), dtype=torch.bfloat16)
+    with pytest.raises(_hip.DiffCacheError, match="no CPU path"):
+        _hip.score(k, q, 0, 16)
+    with pytest.raises(_hip.DiffCacheError):
+        _hip.score_select(k, q, 0, 16, 4)
+
+
+def test_invalid_arguments_are_reported_not_launched():
+    from diffcache_amd import _hip
+    rc = _hip.lib.dc_score_bf16(None, None, None, None, 1, 1, 1, 128, 0, 0, 128, 1, 1, 0, None)
+    assert rc == -22 and b"null pointer" in _hip.lib.dc_last_error()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 255) // 256 * 256
+    rc = _hip.lib.dc_score_bf16(p, p, p, None, 1, 1, 1, 96, 0, 0, 96, 1, 1, 0, None)
+    assert rc == -22 and b"head_dim" in _hip.lib.dc_last_error()
+    rc = _hip.lib.dc_topk_select(p, 8, p, 8, 1, 8, 4, 7, 0, None, p, 1024, None)
+    assert rc == -22 and b"mode" in _hip.lib.dc_last_error()
+    rc = _hip.lib.dc_topk_select(p, 100000, p, 8, 1, 100000, 4, 0, 0, None, p, 16, None)
+    assert rc == -12 and b"workspace" in _hip.lib.dc_last_error()
+
+
+def test_data_layer_option_errors():
+    from diffcache_amd import DiffCacheHIP
+    from diffcache_amd._hip import DiffCacheError
+    with pytest.raises(ValueError, match="Unknown option"):      # lib.rs:579
+        DiffCacheHIP(1, 8, 2, 128, bogus=1)
+    with pytest.raises(AssertionError, match="multiple"):        # lib.rs:294
+        DiffCacheHIP(1, 7, 2, 128)
+    with pytest.raises(DiffCacheError, match="no CPU path"):
+        DiffCacheHIP(1, 8, 2, 128, device="cpu", max_ctx_len=8)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True)
+    assert res.returncode != 0 and "one GPU" in res.stderr
+
+
+# ---------------------------------------------------------------- snapshot codec
+
+def test_varint_known_answers():
+    from diffcache_amd import snapshot
+    assert snapshot._varint(0) == b"\x00"
+    assert snapshot._varint(250) == b"\xfa"
+    assert snapshot._varint(251) == b"\xfb\xfb\x00"
+    assert snapshot._varint(65535) == b"\xfb\xff\xff"
+    assert snapshot._varint(65536) == b"\xfc\x00\x00\x01\x00"
+    assert snapshot._varint(1 << 32) == b"\xfd" + struct.pack("<Q", 1 << 32)
+
+
+def test_snapshot_bytes_of_a_tiny_index(tmp_path):
+    """Hand-assembled bincode of a 2-node, dim-2 index (field order of
+    nsw.rs:64-72, options of nsw.rs:22-31)."""
+    from diffcache_amd import snapshot
+    path = str(tmp_path / "t.idx")
+    keys = np.float32([[1.0, 2.0], [3.0, 4.0]])
+    vals = np.float32([[5.0, 6.0], [7.0, 8.0]])
+    snapshot.write(path, keys, vals, m=16, ef_cons=200, n_max=1000, r_sq=4.0, name="l0",
+                   attn_mass_threshold=0.5, k_check_seq=[100, 300])
+    want = (b"\x02" + b"\x00\x00" + b"\x01\x00"                       # 2 nodes: (id, 0 edges)
+            + b"\x04" + keys.tobytes() + b"\x04" + vals.tobytes()     # Vec<f32> x 2
+            + b"\x10" + b"\xc8" + b"\xfb\xe8\x03"                     # m 16, ef_cons 200, n_max 1000
+            + struct.pack("<f", 4.0) + b"\x02l0" + struct.pack("<f", 0.5)
+            + b"\x02" + b"\x64" + b"\xfb\x2c\x01"                     # k_check_seq [100, 300]
+            + b"\x02" + b"\x02")                                      # dim, num_nodes
+    assert open(path, "rb").read() == want
+    snap = snapshot.read(path)
+    assert np.array_equal(snap["keys"], keys) and np.array_equal(snap["vals"], vals)
+    assert snap["options"]["k_check_seq"] == [100, 300] and snap["options"]["name"] == "l0"
+    assert snap["dim"] == 2 and snap["num_nodes"] == 2
+
+
+def test_snapshot_with_edges_as_the_reference_writes_them(tmp_path):
+    """A file whose nodes carry edge lists (what the reference saves) must load."""
+    from diffcache_amd import snapshot
+    keys = np.float32([[1.0], [2.0], [3.0]])
+    raw = (b"\x03" + b"\x00\x02\x01\x02" + b"\x01\x01\x00" + b"\x02\x00"
+           + b"\x03" + keys.tobytes() + b"\x03" + keys.tobytes()
+           + b"\x10\xc8\x0a" + struct.pack("<f", 4.0) + b"\x01x" + struct.pack("<f", 0.9) + b"\x00"
+           + b"\x01\x03")
+    path = str(tmp_path / "e.idx")
+    open(path, "wb").write(raw)
+    snap = snapshot.read(path, keep_edges=True)
+    assert snap["edges"] == [[1, 2], [0], []]
+    assert np.array_equal(snap["keys"], keys)
+
+
+def test_snapshot_roundtrip_many_nodes(tmp_path):
+    from diffcache_amd import snapshot
+    rng = np.random.default_rng(0)
+    n, dim = 70000, 8                      # crosses the 251 and 65536 varint boundaries
+    keys = rng.standard_normal((n, dim)).astype(np.float32)
+    vals = rng.standard_normal((n, dim)).astype(np.float32)
+    path = str(tmp_path / "big.idx")
+    snapshot.write(path, keys, vals, m=16, ef_cons=200, n_max=n, r_sq=1.5, name="l003b001h002",
+                   attn_mass_threshold=0.9, k_check_seq=[1048576])
+    snap = snapshot.read(path)
+    assert np.array_equal(snap["keys"], keys) and np.array_equal(snap["vals"], vals)
+    assert snap["num_nodes"] == n and snap["options"]["n_max"] == n
