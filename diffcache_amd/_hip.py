@@ -124,7 +124,8 @@ def _store_strides(store: torch.Tensor) -> Tuple[int, int, int]:
 
 
 def alloc_workspace(nbytes: int, device) -> torch.Tensor:
-    return torch.empty((max(int(nbytes), 256) + 255) // 256 * 256, dtype=torch.uint8, device=device)
+    """Zero-filled, 256-byte aligned scratch (the attention counters must start at zero)."""
+    return torch.zeros((max(int(nbytes), 256) + 255) // 256 * 256, dtype=torch.uint8, device=device)
 
 
 # ---------------------------------------------------------------------------

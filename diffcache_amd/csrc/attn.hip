@@ -3,14 +3,17 @@
 // call of src/diffcache/base.py:134-142: the selected rows are read straight
 // from the HBM-resident store instead of being copied into a dense buffer.
 //
-// Grid: one block per (unit, split); a split is a contiguous slice of the
-// unit's attended list [selected | sinks | recent | current token].  Inside a
-// block a group of LPR = HD/8 lanes owns one row at a time (one 16-byte load
-// per lane covers the row) and the G query heads of the GQA group share every
-// row that is loaded.  Three passes over the slice: logits into LDS, a
-// block-wide max / exp / sum per head, then the V accumulation without any
-// rescaling.  Each split writes (m, l, acc) and merge_kernel combines the
-// splits through their log-sum-exp.  Bound by HBM: 2 * HD*2 bytes per row.
+// Grid: one block per (unit, split); a split is a slice of kRowsPerGroup * NG
+// consecutive positions of the unit's attended list [selected | sinks | recent |
+// current token] (64 rows at head_dim 128).  A group of LPR = HD/8 lanes owns one
+// row at a time (one 16-byte load per lane covers the row) and the G query heads
+// of the GQA group share every row that is loaded.  All K and V rows of the
+// slice are requested up front (one memory round trip after the id lookup), the
+// logits stay in registers, the block agrees on a per-head maximum, and each
+// split leaves (m, l, acc) in the workspace; merge_kernel combines the splits
+// through their log-sum-exp.  (Merging in the last block to arrive was tried:
+// the device-scope fence it needs costs far more than a second launch here.)
+// Bound by HBM: 2 * HD*2 bytes per row.
 #include "dc_common.h"
 #include <math.h>
 
@@ -18,30 +21,18 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
-constexpr int kMaxRowsPerSplit = 512;
+constexpr int kRowsPerGroup = 4;
 constexpr uint32_t kNewToken = 0xffffffffu;
-constexpr int kInflight = 4;
 
 struct AttnPlan {
     int rows_per_split;
     int n_splits;
 };
 
-AttnPlan plan_attn(int n_units, int n_total) {
+AttnPlan plan_attn(int hd, int n_total) {
     AttnPlan p;
-    if (n_total <= 0) {
-        p.rows_per_split = 16;
-        p.n_splits = 1;
-        return p;
-    }
-    int want = (1024 + n_units - 1) / (n_units > 0 ? n_units : 1);
-    if (want < 1) want = 1;
-    int rps = (n_total + want - 1) / want;
-    if (rps < 16) rps = 16;
-    if (rps > kMaxRowsPerSplit) rps = kMaxRowsPerSplit;
-    rps = (rps + 15) / 16 * 16;
-    p.rows_per_split = rps;
-    p.n_splits = (n_total + rps - 1) / rps;
+    p.rows_per_split = (kThreads / (hd / 8)) * kRowsPerGroup;
+    p.n_splits = n_total > 0 ? (n_total + p.rows_per_split - 1) / p.rows_per_split : 1;
     return p;
 }
 
@@ -49,15 +40,16 @@ template <int HD, int G>
 __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint32_t *__restrict__ idx, const uint16_t *__restrict__ new_k,
-    const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml,
-    int n_h, int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo,
-    int n_recent, int n_total, int rows_per_split, int n_splits, int64_t ksb, int64_t ksh,
-    int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale) {
+    const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml, int n_h,
+    int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
+    int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
+    int64_t vsr, float scale) {
     constexpr int LPR = HD / 8;
     constexpr int NG = kThreads / LPR;  // row groups per block
-    __shared__ uint32_t s_rows[kMaxRowsPerSplit];
-    __shared__ float s_logit[G][kMaxRowsPerSplit];
+    constexpr int R = kRowsPerGroup;
+    constexpr int ROWS = NG * R;
     __shared__ float s_red[kWaves][G];
+    __shared__ float s_l[kWaves][G];
     __shared__ float s_acc[kWaves][G * HD];
 
     const int unit = blockIdx.x / n_splits;
@@ -65,71 +57,78 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const int b = unit / n_h, h = unit % n_h;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gid = tid / LPR, col = tid % LPR;
+    const int r0 = split * ROWS;
 
-    const int r0 = split * rows_per_split;
-    int n = n_total - r0;
-    n = n < rows_per_split ? n : rows_per_split;
-    n = n < 0 ? 0 : n;
-
-    // ---- pass 0: physical row of every list position of this slice ----
-    for (int j = tid; j < n; j += kThreads) {
-        const int vj = r0 + j;
-        uint32_t row;
-        if (vj < n_idx) row = (uint32_t)(region_lo + idx[(int64_t)unit * idx_stride + vj]);
-        else if (vj < n_idx + n_sink) row = (uint32_t)(vj - n_idx);
-        else if (vj < n_idx + n_sink + n_recent) row = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
-        else row = kNewToken;
-        s_rows[j] = row;
+    // physical rows of this group's list positions
+    uint32_t row[R];
+    bool ok[R];
+#pragma unroll
+    for (int t = 0; t < R; ++t) {
+        const int vj = r0 + t * NG + gid;
+        ok[t] = vj < n_total;
+        uint32_t r = 0;
+        if (ok[t]) {
+            if (vj < n_idx) r = (uint32_t)(region_lo + idx[(int64_t)unit * idx_stride + vj]);
+            else if (vj < n_idx + n_sink) r = (uint32_t)(vj - n_idx);
+            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
+            else r = kNewToken;
+        }
+        row[t] = r;
     }
-
     float qf[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const uint16_t *qp = Q + ((int64_t)unit * G + g) * HD + col * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qf[g][i] = dc_bf16_to_f32(qp[i]);
+        const uint4 w = *reinterpret_cast<const uint4 *>(Q + ((int64_t)unit * G + g) * HD + col * 8);
+        qf[g][0] = dc_bf16_lo(w.x);
+        qf[g][1] = dc_bf16_hi(w.x);
+        qf[g][2] = dc_bf16_lo(w.y);
+        qf[g][3] = dc_bf16_hi(w.y);
+        qf[g][4] = dc_bf16_lo(w.z);
+        qf[g][5] = dc_bf16_hi(w.z);
+        qf[g][6] = dc_bf16_lo(w.w);
+        qf[g][7] = dc_bf16_hi(w.w);
     }
-    __syncthreads();
-
     const uint16_t *Ku = K + b * ksb + h * ksh + col * 8;
     const uint16_t *Vu = V + b * vsb + h * vsh + col * 8;
-    const uint16_t *nk = new_k ? new_k + (int64_t)unit * HD + col * 8 : nullptr;
-    const uint16_t *nv = new_v ? new_v + (int64_t)unit * HD + col * 8 : nullptr;
+    const uint16_t *nk = new_k ? new_k + (int64_t)unit * HD + col * 8 : Ku;
+    const uint16_t *nv = new_v ? new_v + (int64_t)unit * HD + col * 8 : Vu;
 
-    // ---- pass 1: scaled logits of every (head, row) into LDS ----
-    for (int base = 0; base < n; base += kInflight * NG) {
-        uint4 w[kInflight];
+    // every K and V row of the slice is requested before any is used
+    uint4 kw[R], vw[R];
 #pragma unroll
-        for (int t = 0; t < kInflight; ++t) {
-            int j = base + t * NG + gid;
-            j = j < n ? j : n - 1;
-            const uint32_t row = s_rows[j];
-            const uint16_t *p = (row == kNewToken) ? nk : Ku + (int64_t)row * ksr;
-            w[t] = *reinterpret_cast<const uint4 *>(p);
-        }
-#pragma unroll
-        for (int t = 0; t < kInflight; ++t) {
-            const int j = base + t * NG + gid;
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                float p = dc_group_sum<LPR>(dc_dot8(w[t], qf[g], 0.f));
-                if (col == g % LPR && j < n) s_logit[g][j] = p * scale;
-            }
-        }
+    for (int t = 0; t < R; ++t) {
+        const uint16_t *pk = (row[t] == kNewToken) ? nk : Ku + (int64_t)row[t] * ksr;
+        kw[t] = *reinterpret_cast<const uint4 *>(pk);
     }
-    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < R; ++t) {
+        const uint16_t *pv = (row[t] == kNewToken) ? nv : Vu + (int64_t)row[t] * vsr;
+        vw[t] = *reinterpret_cast<const uint4 *>(pv);
+    }
 
-    // ---- pass 2: per-head max, exponentials, sum ----
-    float m[G], l[G];
+    // scaled logits, in registers: x[t][g] is known to every lane of the group
+    float x[R][G];
+    float mloc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) mloc[g] = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < R; ++t)
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float v = dc_group_sum<LPR>(dc_dot8(kw[t], qf[g], 0.f)) * scale;
+            x[t][g] = ok[t] ? v : -INFINITY;
+            mloc[g] = fmaxf(mloc[g], x[t][g]);
+        }
+    // per-head maximum over the block
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        float v = -INFINITY;
-        for (int j = tid; j < n; j += kThreads) v = fmaxf(v, s_logit[g][j]);
+        float v = mloc[g];
 #pragma unroll
-        for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d, 64));
+        for (int off = LPR; off < 64; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
         if (lane == 0) s_red[wave][g] = v;
     }
     __syncthreads();
+    float m[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         float v = s_red[0][g];
@@ -137,73 +136,46 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
         for (int w2 = 1; w2 < kWaves; ++w2) v = fmaxf(v, s_red[w2][g]);
         m[g] = v;
     }
-    __syncthreads();
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float s = 0.f;
-        for (int j = tid; j < n; j += kThreads) {
-            float p = __expf(s_logit[g][j] - m[g]);
-            s_logit[g][j] = p;
-            s += p;
-        }
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) s += __shfl_xor(s, d, 64);
-        if (lane == 0) s_red[wave][g] = s;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float s = s_red[0][g];
-#pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) s += s_red[w2][g];
-        l[g] = s;
-    }
 
-    // ---- pass 3: acc[g] += p[g][row] * V[row] ----
+    // p = exp(x - m), acc[g] += p * V
     float acc[G][8];
+    float lloc[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) {
+        lloc[g] = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-    for (int base = 0; base < n; base += kInflight * NG) {
-        uint4 w[kInflight];
+    }
 #pragma unroll
-        for (int t = 0; t < kInflight; ++t) {
-            int j = base + t * NG + gid;
-            j = j < n ? j : n - 1;
-            const uint32_t row = s_rows[j];
-            const uint16_t *p = (row == kNewToken) ? nv : Vu + (int64_t)row * vsr;
-            w[t] = *reinterpret_cast<const uint4 *>(p);
-        }
+    for (int t = 0; t < R; ++t) {
+        const float v[8] = {dc_bf16_lo(vw[t].x), dc_bf16_hi(vw[t].x), dc_bf16_lo(vw[t].y),
+                            dc_bf16_hi(vw[t].y), dc_bf16_lo(vw[t].z), dc_bf16_hi(vw[t].z),
+                            dc_bf16_lo(vw[t].w), dc_bf16_hi(vw[t].w)};
 #pragma unroll
-        for (int t = 0; t < kInflight; ++t) {
-            const int j = base + t * NG + gid;
-            const bool ok = j < n;
-            const int jj = ok ? j : 0;
-            float v[8] = {dc_bf16_lo(w[t].x), dc_bf16_hi(w[t].x), dc_bf16_lo(w[t].y),
-                          dc_bf16_hi(w[t].y), dc_bf16_lo(w[t].z), dc_bf16_hi(w[t].z),
-                          dc_bf16_lo(w[t].w), dc_bf16_hi(w[t].w)};
+        for (int g = 0; g < G; ++g) {
+            const float p = ok[t] ? __expf(x[t][g] - m[g]) : 0.f;
+            lloc[g] += p;
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const float p = ok ? s_logit[g][jj] : 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
-            }
+            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
         }
     }
 
-    // ---- reduce over the row groups: inside the wave, then across waves ----
+    // reduce over the row groups: inside the wave, then across waves
 #pragma unroll
     for (int off = LPR; off < 64; off <<= 1)
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int g = 0; g < G; ++g) {
+            lloc[g] += __shfl_xor(lloc[g], off, 64);
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[g][i] += __shfl_xor(acc[g][i], off, 64);
+        }
     if (lane < LPR) {
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int g = 0; g < G; ++g) {
+            if (col == 0) s_l[wave][g] = lloc[g];
 #pragma unroll
             for (int i = 0; i < 8; ++i) s_acc[wave][g * HD + col * 8 + i] = acc[g][i];
+        }
     }
     __syncthreads();
     const int64_t slot = (int64_t)unit * n_splits + split;
@@ -213,39 +185,76 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
         for (int w2 = 1; w2 < kWaves; ++w2) s += s_acc[w2][o];
         ws_acc[slot * (G * HD) + o] = s;
     }
+    if (tid < G) {
+        float l = s_l[0][tid];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        if (tid == g) {
-            ws_ml[(slot * G + g) * 2 + 0] = m[g];
-            ws_ml[(slot * G + g) * 2 + 1] = l[g];
-        }
+        for (int w2 = 1; w2 < kWaves; ++w2) l += s_l[w2][tid];
+        float mm = s_red[0][tid];
+#pragma unroll
+        for (int w2 = 1; w2 < kWaves; ++w2) mm = fmaxf(mm, s_red[w2][tid]);
+        ws_ml[(slot * G + tid) * 2 + 0] = mm;
+        ws_ml[(slot * G + tid) * 2 + 1] = l;
     }
+
 }
 
-// out[u, g, :] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s
-__global__ void merge_kernel(const float *__restrict__ ws_acc, const float *__restrict__ ws_ml,
-                             uint16_t *__restrict__ out, float *__restrict__ lse, int group, int hd,
-                             int n_splits) {
+// out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block
+// per (unit, head), one thread per output column.
+__global__ __launch_bounds__(256) void merge_kernel(const float *__restrict__ ws_acc,
+                                                    const float *__restrict__ ws_ml,
+                                                    uint16_t *__restrict__ out, float *__restrict__ lse,
+                                                    int group, int hd, int n_splits) {
+    __shared__ float s_w[256];
+    __shared__ float s_red[4];
     const int ug = blockIdx.x;  // unit * group + g
     const int unit = ug / group, g = ug % group;
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s)
-        M = fmaxf(M, ws_ml[(((int64_t)unit * n_splits + s) * group + g) * 2]);
-    float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float *ml = ws_ml + (((int64_t)unit * n_splits + s) * group + g) * 2;
-        if (ml[1] > 0.f) L += __expf(ml[0] - M) * ml[1];
-    }
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float a = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const int64_t slot = (int64_t)unit * n_splits + s;
-            const float *ml = ws_ml + (slot * group + g) * 2;
-            if (ml[1] > 0.f) a += __expf(ml[0] - M) * ws_acc[(slot * group + g) * hd + d];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+    const float *ml = ws_ml + ((int64_t)unit * n_splits * group + g) * 2;  // split s at ml + s*group*2
+    float acc = 0.f, M = -INFINITY, L = 0.f;
+    // splits are folded in chunks of at most blockDim.x with a running maximum
+    for (int s0 = 0; s0 < n_splits; s0 += blockDim.x) {
+        const int sp = s0 + tid;
+        float m = -INFINITY, l = 0.f;
+        if (sp < n_splits) {
+            m = ml[(int64_t)sp * group * 2];
+            l = ml[(int64_t)sp * group * 2 + 1];
+            if (!(l > 0.f)) m = -INFINITY;
         }
-        out[(int64_t)ug * hd + d] = dc_f32_to_bf16(L > 0.f ? a / L : 0.f);
+        float cm = m;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) cm = fmaxf(cm, __shfl_xor(cm, d, 64));
+        if (lane == 0) s_red[wave] = cm;
+        __syncthreads();
+        cm = s_red[0];
+        for (int w = 1; w < nw; ++w) cm = fmaxf(cm, s_red[w]);
+        __syncthreads();
+        const float Mn = fmaxf(M, cm);
+        const float rescale = (M > -INFINITY) ? __expf(M - Mn) : 0.f;
+        const float w = (m > -INFINITY) ? __expf(m - Mn) : 0.f;
+        s_w[tid] = w;
+        float cl = w * l;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) cl += __shfl_xor(cl, d, 64);
+        if (lane == 0) s_red[wave] = cl;
+        __syncthreads();
+        cl = s_red[0];
+        for (int w2 = 1; w2 < nw; ++w2) cl += s_red[w2];
+        L = L * rescale + cl;
+        acc *= rescale;
+        M = Mn;
+        const int cnt = (n_splits - s0) < (int)blockDim.x ? (n_splits - s0) : (int)blockDim.x;
+        for (int d = tid; d < hd; d += blockDim.x) {
+            // every thread owns one column when hd <= blockDim.x (the launch guarantees it)
+            float a = 0.f;
+            const float *pa = ws_acc + (((int64_t)unit * n_splits + s0) * group + g) * hd + d;
+#pragma unroll 8
+            for (int j = 0; j < cnt; ++j) a = fmaf(s_w[j], pa[(int64_t)j * group * hd], a);
+            acc += a;
+        }
+        __syncthreads();
     }
-    if (lse && threadIdx.x == 0) lse[ug] = L > 0.f ? M + logf(L) : -INFINITY;
+    if (tid < hd) out[(int64_t)ug * hd + tid] = dc_f32_to_bf16(L > 0.f ? acc / L : 0.f);
+    if (lse && tid == 0) lse[ug] = L > 0.f ? M + logf(L) : -INFINITY;
 }
 
 template <int HD>
@@ -269,19 +278,37 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
     if (out_v) *reinterpret_cast<uint4 *>(out_v + dst) = *reinterpret_cast<const uint4 *>(V + src);
 }
 
+struct AttnWs {
+    float *acc, *ml;
+    size_t bytes;
+};
+
+AttnWs carve_attn(void *base, int n_units, int group, int hd, int n_splits) {
+    AttnWs w;
+    char *p = (char *)base;
+    size_t off = 0;
+    const size_t slots = (size_t)(n_units > 0 ? n_units : 0) * (size_t)n_splits;
+    w.acc = (float *)(p + off);
+    off += dc_align_up(slots * group * hd * 4, 256);
+    w.ml = (float *)(p + off);
+    off += dc_align_up(slots * group * 2 * 4, 256);
+    w.bytes = off;
+    return w;
+}
+
 template <int HD>
 int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const uint16_t *k,
                 const uint16_t *v, const uint32_t *idx, const uint16_t *new_k,
-                const uint16_t *new_v, float *ws_acc, float *ws_ml, int n_h, int n_idx,
+                const uint16_t *new_v, const AttnWs &w, int n_h, int n_idx,
                 int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-                int n_total, AttnPlan plan, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
+                int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
                 int64_t vsh, int64_t vsr, float scale) {
 #define DC_ATTN_CASE(GG)                                                                           \
     case GG:                                                                                       \
         hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, q, k, v, idx, \
-                           new_k, new_v, ws_acc, ws_ml, n_h, n_idx, idx_stride, region_lo, n_sink, \
-                           recent_lo, n_recent, n_total, plan.rows_per_split, plan.n_splits, ksb,  \
-                           ksh, ksr, vsb, vsh, vsr, scale);                                        \
+                           new_k, new_v, w.acc, w.ml, n_h, n_idx, idx_stride,                      \
+                           region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, ksb, ksh,    \
+                           ksr, vsb, vsh, vsr, scale);                                             \
         return 0;
     switch (group) {
         DC_ATTN_CASE(1)
@@ -299,19 +326,9 @@ int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const u
 
 }  // namespace
 
-// Upper bound of plan_attn(n_units, n).n_splits over every n <= n_total, so that a
-// workspace sized for the longest attended list also serves shorter ones.
-static int max_splits(int n_units, int n_total) {
-    int want = (1024 + n_units - 1) / (n_units > 0 ? n_units : 1);
-    int by_cap = (n_total + kMaxRowsPerSplit - 1) / kMaxRowsPerSplit;
-    int m = want > by_cap ? want : by_cap;
-    return m < 1 ? 1 : m;
-}
-
 extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attended) {
-    if (n_units <= 0 || group <= 0 || hd <= 0) return 256;
-    size_t slots = (size_t)n_units * max_splits(n_units, n_rows_attended);
-    return dc_align_up(slots * group * hd * 4, 256) + dc_align_up(slots * group * 2 * 4, 256);
+    if (n_units <= 0 || group <= 0 || hd < 8) return 256;
+    return carve_attn(nullptr, n_units, group, hd, plan_attn(hd, n_rows_attended).n_splits).bytes;
 }
 
 extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
@@ -341,38 +358,37 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
     const int n_units = n_b * n_h;
     if (n_units == 0) return DC_OK;
     const int n_total = n_idx + n_sink + n_recent + (new_k ? 1 : 0);
-    AttnPlan plan = plan_attn(n_units, n_total);
-    const size_t slots = (size_t)n_units * plan.n_splits;
-    const size_t need = dc_align_up(slots * group * hd * 4, 256) + dc_align_up(slots * group * 2 * 4, 256);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "dc_gather_attn_bf16: workspace must be non-null and 256-byte aligned");
-    if (workspace_bytes < need) {
-        dc_set_error("dc_gather_attn_bf16: workspace %zu bytes < %zu needed", workspace_bytes, need);
+    const AttnPlan plan = plan_attn(hd, n_total);
+    const AttnWs w = carve_attn(workspace, n_units, group, hd, plan.n_splits);
+    if (workspace_bytes < w.bytes) {
+        dc_set_error("dc_gather_attn_bf16: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
         return DC_ENOMEM;
     }
-    float *ws_acc = (float *)workspace;
-    float *ws_ml = (float *)((char *)workspace + dc_align_up(slots * group * hd * 4, 256));
+    DC_REQUIRE((int64_t)n_units * plan.n_splits < (1ll << 31), "dc_gather_attn_bf16: grid too large");
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid((unsigned)slots);
+    dim3 grid((unsigned)((size_t)n_units * plan.n_splits));
     int rc;
     const uint16_t *q16 = (const uint16_t *)q, *k16 = (const uint16_t *)k, *v16 = (const uint16_t *)v;
     const uint16_t *nk16 = (const uint16_t *)new_k, *nv16 = (const uint16_t *)new_v;
+    uint16_t *o16 = (uint16_t *)out;
     if (hd == 64)
-        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, ws_acc, ws_ml, n_h, n_idx,
-                             idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total, plan,
-                             ksb, ksh, ksr, vsb, vsh, vsr, scale);
+        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+                             idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
+                             plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else if (hd == 128)
-        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, ws_acc, ws_ml, n_h,
-                              n_idx, idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
+                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else
-        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, ws_acc, ws_ml, n_h,
-                              n_idx, idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
+                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     DC_REQUIRE(rc == 0, "dc_gather_attn_bf16: unsupported group %d", group);
     DC_CHECK_LAUNCH("dc_gather_attn_bf16(attn)");
-    hipLaunchKernelGGL(merge_kernel, dim3((unsigned)(n_units * group)), dim3(hd < 256 ? hd : 256), 0,
-                       st, ws_acc, ws_ml, (uint16_t *)out, lse, group, hd, plan.n_splits);
+    hipLaunchKernelGGL(merge_kernel, dim3((unsigned)(n_units * group)), dim3(hd), 0, st, w.acc, w.ml, o16,
+                       lse, group, hd, plan.n_splits);
     DC_CHECK_LAUNCH("dc_gather_attn_bf16(merge)");
     return DC_OK;
 }
