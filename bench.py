@@ -118,8 +118,15 @@ def main() -> int:
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
     ap.add_argument("--mode", default="ref_dist", choices=["ref_dist", "ip"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--fused", action="store_true",
-                    help="time dc_decode_layer (one call per layer) instead of the split calls")
+    ap.add_argument("--split", action="store_true",
+                    help="issue the scan, select and attention as separate C calls with an event between "
+                         "each (per-stage breakdown) instead of one dc_decode_layer call per layer")
+    ap.add_argument("--event-stride", type=int, default=4,
+                    help="one-call path: time the scan kernel in place on every N-th layer")
+    ap.add_argument("--streams", type=int, default=1,
+                    help="pipeline the batch as this many independent micro-batches, one HIP stream each "
+                         "(the units of a layer are independent, so one micro-batch's select/attention "
+                         "overlaps the other's scan)")
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
@@ -154,57 +161,92 @@ def main() -> int:
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t_gen
 
-    scores = torch.empty((n_units, region), dtype=torch.float32, device=dev)
-    idx = torch.empty((n_units, budget), dtype=torch.int32, device=dev)
-    out = torch.empty((b, hq, hd), dtype=torch.bfloat16, device=dev)
-    hist = hip.new_hist(n_units, dev)
-    ws_topk = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(n_units, region, budget), dev)
-    ws_attn = hip.alloc_workspace(hip.lib.dc_attn_workspace_bytes(n_units, grp, hd, attended), dev)
-    ws_layer = hip.alloc_workspace(hip.layer_workspace_bytes(n_units, region, budget, grp, hd, attended), dev)
-    ws_sel = hip.alloc_workspace(hip.score_select_workspace_bytes(n_units, region, budget), dev)
+    if args.streams < 1 or b % args.streams != 0:
+        print("bench.py: --streams must divide the batch size", file=sys.stderr)
+        return 2
+    args.fused = not args.split
+
+    class Pipe:
+        """One micro-batch: its slice of every layer's tensors, its buffers, its stream."""
+
+        def __init__(self, b0, b1):
+            self.nb = b1 - b0
+            self.n_units = self.nb * hkv
+            self.layers = [(k[b0:b1], v[b0:b1], q[b0:b1], nk[b0:b1], nv[b0:b1]) for (k, v, q, nk, nv) in layers]
+            nu = self.n_units
+            self.scores = torch.empty((nu, region), dtype=torch.float32, device=dev) if args.dense else None
+            self.idx = torch.empty((nu, budget), dtype=torch.int32, device=dev)
+            self.out = torch.empty((self.nb, hq, hd), dtype=torch.bfloat16, device=dev)
+            self.hist = hip.new_hist(nu, dev)
+            self.ws_topk = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, region, budget), dev)
+            self.ws_attn = hip.alloc_workspace(hip.lib.dc_attn_workspace_bytes(nu, grp, hd, attended), dev)
+            self.ws_layer = hip.alloc_workspace(hip.layer_workspace_bytes(nu, region, budget, grp, hd, attended), dev)
+            self.ws_sel = hip.alloc_workspace(hip.score_select_workspace_bytes(nu, region, budget), dev)
+            self.stream = torch.cuda.Stream(device=dev)     # default priority
+            self.clean = False
+
+        def layer(self, l, ev=None):
+            k, v, q, nk, nv = self.layers[l]
+            nu = self.n_units
+            if args.fused:
+                hip.decode_layer(q, k, v, sink, hi, recent, budget, self.scores, self.idx, self.out,
+                                 self.ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY,
+                                 select_state_ready=self.clean and not args.dense,
+                                 scan_events=None if ev is None or l % args.event_stride else
+                                 (ev[4 * l], ev[4 * l + 1]))
+                self.clean = True
+                return
+            if args.dense:
+                self.hist.zero_()
+            elif not self.clean:
+                hip.select_state_init(nu, region, budget, self.ws_sel)
+                self.clean = True   # dc_sparse_select(reinit) keeps it so from here on
+            if ev is not None:
+                ev[4 * l + 0].record()
+            if args.dense:
+                hip.score(k, q, lo, region, mode, q_group=grp, scores=self.scores, hist=self.hist)
+            else:
+                hip.score_prune(k, q, lo, region, budget, self.ws_sel, mode, q_group=grp)
+            if ev is not None:
+                ev[4 * l + 1].record()
+            if args.dense:
+                hip.topk_select(self.scores, budget, mode, hip.ORDER_ANY, hist=self.hist, idx_out=self.idx,
+                                workspace=self.ws_topk)
+            else:
+                hip.sparse_select(self.idx, nu, region, budget, self.ws_sel, mode, hip.ORDER_ANY, reinit=True)
+            if ev is not None:
+                ev[4 * l + 2].record()
+            hip.gather_attn(q, k, v, self.idx, k_eff, lo, sink, hi, recent, nk, nv, out=self.out,
+                            workspace=self.ws_attn)
+            if ev is not None:
+                ev[4 * l + 3].record()
+
+    per = b // args.streams
+    pipes = [Pipe(i * per, (i + 1) * per) for i in range(args.streams)]
 
     def new_events(count):
         return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
 
-    state = {"clean": False}
-
-    def step(ev=None):
-        """One decode step: every layer, in order, on the current stream."""
+    def step(evs=None):
+        """One decode step: every layer in order; the micro-batches are independent of
+        each other and each runs its layers in order on its own stream."""
         for l in range(L):
-            k, v, q, nk, nv = layers[l]
-            if args.fused:
-                hip.decode_layer(q, k, v, sink, hi, recent, budget, scores if args.dense else None, idx,
-                                 out, ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY)
-                continue
-            if args.dense:
-                hist.zero_()
-            elif not state["clean"]:
-                hip.select_state_init(n_units, region, budget, ws_sel)
-                state["clean"] = True   # dc_sparse_select(reinit) keeps it so from here on
-            if ev is not None:
-                ev[4 * l + 0].record()
-            if args.dense:
-                hip.score(k, q, lo, region, mode, q_group=grp, scores=scores, hist=hist)
-            else:
-                hip.score_prune(k, q, lo, region, budget, ws_sel, mode, q_group=grp)
-            if ev is not None:
-                ev[4 * l + 1].record()
-            if args.dense:
-                hip.topk_select(scores, budget, mode, hip.ORDER_ANY, hist=hist, idx_out=idx,
-                                workspace=ws_topk)
-            else:
-                hip.sparse_select(idx, n_units, region, budget, ws_sel, mode, hip.ORDER_ANY, reinit=True)
-            if ev is not None:
-                ev[4 * l + 2].record()
-            hip.gather_attn(q, k, v, idx, k_eff, lo, sink, hi, recent, nk, nv, out=out,
-                            workspace=ws_attn)
-            if ev is not None:
-                ev[4 * l + 3].record()
+            for pi, pipe in enumerate(pipes):
+                with torch.cuda.stream(pipe.stream):
+                    pipe.layer(l, None if evs is None else evs[pi])
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    events = [new_events(4 * L) for _ in range(args.steps)] if not args.fused else None
+    events = [[new_events(4 * L) for _ in pipes] for _ in range(args.steps)]
+    if args.fused:
+        # torch creates the native event on first record; the C side needs the handle
+        for per_step in events:
+            for pi, evs in enumerate(per_step):
+                for l in range(0, L, args.event_stride):
+                    evs[4 * l].record(pipes[pi].stream)
+                    evs[4 * l + 1].record(pipes[pi].stream)
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(args.steps):
         step(None if events is None else events[s])
@@ -215,18 +257,23 @@ def main() -> int:
     # per-kernel durations from the events of the timed region
     stage_us = None
     score_ms = None
-    if events is not None:
-        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in events for l in range(L)]
-        se = [e[4 * l + 1].elapsed_time(e[4 * l + 2]) for e in events for l in range(L)]
-        at = [e[4 * l + 2].elapsed_time(e[4 * l + 3]) for e in events for l in range(L)]
+    flat = [e for per_step in events for e in per_step]
+    if args.fused:
+        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(0, L, args.event_stride)]
+        score_ms = sum(sc) / len(sc)
+        stage_us = {"score": score_ms * 1e3, "timed_launches": len(sc)}
+    else:
+        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(L)]
+        se = [e[4 * l + 1].elapsed_time(e[4 * l + 2]) for e in flat for l in range(L)]
+        at = [e[4 * l + 2].elapsed_time(e[4 * l + 3]) for e in flat for l in range(L)]
         score_ms = sum(sc) / len(sc)
         stage_us = {"score": score_ms * 1e3, "select": sum(se) / len(se) * 1e3,
-                    "attn": sum(at) / len(at) * 1e3}
+                    "attn": sum(at) / len(at) * 1e3, "timed_launches": len(sc)}
 
     unit_bytes = algorithmic_bytes_per_unit(region, k_eff + sink + recent, grp, hd)
     step_bytes = unit_bytes * n_units * L
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
-    score_bytes = n_units * region * hd * 2          # K rows streamed by one score launch
+    score_bytes = (n_units // args.streams) * region * hd * 2   # K rows streamed by one scan launch
     roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
                 "traffic": None, "kernel": "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
                 "algorithmic_bytes_per_launch": score_bytes}
@@ -247,8 +294,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": cfg["desc"], "key_mode": args.mode,
-                   "call_path": ("dc_decode_layer" if args.fused else
+        "config": {"workload": cfg["desc"], "key_mode": args.mode, "streams": args.streams,
+                   "call_path": ("dc_decode_layer" + (" (dense scores)" if args.dense else "") if args.fused else
                                  "dc_score_bf16/dc_topk_select/dc_gather_attn_bf16" if args.dense else
                                  "dc_select_state_init/dc_score_prune_bf16/dc_sparse_select/dc_gather_attn_bf16")},
         "step_hbm_gbps": step_gbps,

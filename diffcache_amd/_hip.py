@@ -48,6 +48,8 @@ class LayerArgs(C.Structure):
         ("n_b", C.c_int), ("n_h", C.c_int), ("group", C.c_int), ("hd", C.c_int),
         ("n_sink", C.c_int), ("n_recent", C.c_int), ("budget", C.c_int),
         ("mode", C.c_int), ("order", C.c_int), ("scale", C.c_float),
+        ("select_state_ready", C.c_int),
+        ("ev_scan_begin", C.c_void_p), ("ev_scan_end", C.c_void_p),
     ]
 
 
@@ -328,8 +330,11 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
                  idx_out: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor,
                  new_k: Optional[torch.Tensor] = None, new_v: Optional[torch.Tensor] = None,
                  lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
-                 order: int = ORDER_ANY, scale: Optional[float] = None) -> torch.Tensor:
-    """score -> select -> attend for one layer, enqueued on the current stream."""
+                 order: int = ORDER_ANY, scale: Optional[float] = None,
+                 select_state_ready: bool = False,
+                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None) -> torch.Tensor:
+    """score -> select -> attend for one layer, enqueued on the current stream.
+    ``select_state_ready``: see dc_layer_args in the header (skips the init kernel)."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
         raise DiffCacheError("K and V stores must share their strides")
@@ -353,6 +358,10 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
     a.n_sink, a.n_recent, a.budget = n_sink, n_recent, budget
     a.mode, a.order = mode, order
     a.scale = 1.0 / math.sqrt(hd) if scale is None else scale
+    a.select_state_ready = 1 if select_state_ready else 0
+    if scan_events is not None:
+        # torch creates the underlying event lazily: both must have been recorded once before
+        a.ev_scan_begin, a.ev_scan_end = scan_events[0].cuda_event, scan_events[1].cuda_event
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
 

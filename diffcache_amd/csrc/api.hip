@@ -88,19 +88,30 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
     if (k_eff > 0 && !a->scores) {
         // no dense scores wanted: streaming score + select
-        rc = dc_score_select_bf16(k_region, a->q, a->idx_out, a->idx_unit_stride, a->n_b, a->n_h, region,
-                                  a->hd, a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride,
-                                  a->group, a->budget, a->mode, a->order, w.topk, w.topk_bytes, stream);
+        if (!a->select_state_ready) {
+            rc = dc_select_state_init(n_units, region, a->budget, w.topk, w.topk_bytes, stream);
+            if (rc) return rc;
+        }
+        if (a->ev_scan_begin) (void)hipEventRecord((hipEvent_t)a->ev_scan_begin, st);
+        rc = dc_score_prune_bf16(k_region, a->q, a->n_b, a->n_h, region, a->hd, a->kv_batch_stride,
+                                 a->kv_head_stride, a->kv_row_stride, a->group, a->budget, a->mode, w.topk,
+                                 w.topk_bytes, stream);
+        if (rc) return rc;
+        if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
+        rc = dc_sparse_select(a->idx_out, a->idx_unit_stride, n_units, region, a->budget, a->mode, a->order,
+                              1, w.topk, w.topk_bytes, stream);
         if (rc) return rc;
     } else if (k_eff > 0) {
         const int64_t n = (int64_t)n_units * DC_HIST_BINS;
         hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                            w.hist, n);
         DC_CHECK_LAUNCH("dc_decode_layer(zero)");
+        if (a->ev_scan_begin) (void)hipEventRecord((hipEvent_t)a->ev_scan_begin, st);
         rc = dc_score_bf16(k_region, a->q, a->scores, w.hist, a->n_b, a->n_h, region, a->hd,
                            a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride,
                            a->scores_unit_stride, a->group, a->mode, stream);
         if (rc) return rc;
+        if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
         rc = dc_topk_select(a->scores, a->scores_unit_stride, a->idx_out, a->idx_unit_stride, n_units,
                             region, a->budget, a->mode, a->order, w.hist, w.topk, w.topk_bytes, stream);
         if (rc) return rc;

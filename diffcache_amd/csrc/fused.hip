@@ -204,15 +204,13 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
     __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
     __shared__ uint32_t sres[4];
     __shared__ uint32_t smisc[2];
-    __shared__ uint32_t s_tb, s_cless, s_win, s_cand;
+    __shared__ uint32_t s_tb, s_cless;
     __shared__ uint32_t lck[kCandLds], lci[kCandLds];  // candidates stay in LDS when they fit
     const int unit = blockIdx.x;
     const int tid = threadIdx.x;
     if (tid == 0) {
         s_tb = DC_HIST_BINS;
         s_cless = 0;
-        s_win = 0;
-        s_cand = 0;
     }
     uint32_t bins[4];
     {
@@ -250,9 +248,11 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
     uint32_t *io = idx_out + (int64_t)unit * idx_stride;
     uint32_t *ko = sel_keys ? sel_keys + (int64_t)unit * k_eff : nullptr;
 
-    const int lane = tid & 63;
-    const unsigned long long lt = (1ull << lane) - 1ull;
-    constexpr int kBatch = 4;  // survivor loads in flight per thread
+    // Survivors are taken 16 per thread at a time: classify into bit masks, one
+    // block-wide scan of the packed (member, candidate) counts, then every thread
+    // writes to its own range -- no atomics on the output cursors.
+    constexpr int kBatch = 16;
+    uint32_t win_base = 0, cand_base = 0;
     for (uint32_t i0 = 0; i0 < n_s; i0 += kBatch * kFinalThreads) {
         uint2 p[kBatch];
 #pragma unroll
@@ -261,41 +261,41 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
             p[j] = make_uint2(0u, 0u);
             if (i < n_s) p[j] = su[i];
         }
+        uint32_t keys[kBatch];
+        uint32_t wmask = 0, cmask = 0;
 #pragma unroll
         for (int j = 0; j < kBatch; ++j) {
             const uint32_t i = i0 + j * kFinalThreads + tid;
             uint32_t key = 0, bucket = 0xffffffffu;
-            const uint32_t id = p[j].x;
             if (i < n_s) dc_key_bucket(__uint_as_float(p[j].y), mode, key, bucket);
-            // one LDS atomic per wave and list
-            const bool is_win = bucket < tb, is_cand = bucket == tb;
-            const unsigned long long mw = __ballot(is_win), mc = __ballot(is_cand);
-            if (mw) {
-                uint32_t base = 0;
-                if (lane == 0) base = atomicAdd(&s_win, (uint32_t)__popcll(mw));
-                base = __shfl(base, 0, 64);
-                const uint32_t slot = base + __popcll(mw & lt);
-                if (is_win && slot < kk) {
-                    io[slot] = id;
-                    if (ko) ko[slot] = key;
+            keys[j] = key;
+            if (bucket < tb) wmask |= 1u << j;
+            else if (bucket == tb) cmask |= 1u << j;
+        }
+        uint32_t tot;
+        const uint32_t ex = block_excl_scan<kFinalThreads>(__popc(wmask) | (__popc(cmask) << 16), wtot, &tot);
+        uint32_t wpos = win_base + (ex & 0xffffu), cpos = cand_base + (ex >> 16);
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            if (wmask & (1u << j)) {
+                if (wpos < kk) {
+                    io[wpos] = p[j].x;
+                    if (ko) ko[wpos] = keys[j];
                 }
-            }
-            if (mc) {
-                uint32_t base = 0;
-                if (lane == 0) base = atomicAdd(&s_cand, (uint32_t)__popcll(mc));
-                base = __shfl(base, 0, 64);
-                const uint32_t slot = base + __popcll(mc & lt);
-                if (is_cand) {
-                    if (slot < (uint32_t)kCandLds) {
-                        lck[slot] = key;
-                        lci[slot] = id;
-                    } else if (slot < (uint32_t)n_rows) {
-                        ck[slot] = key;
-                        ci[slot] = id;
-                    }
+                ++wpos;
+            } else if (cmask & (1u << j)) {
+                if (cpos < (uint32_t)kCandLds) {
+                    lck[cpos] = keys[j];
+                    lci[cpos] = p[j].x;
+                } else if (cpos < (uint32_t)n_rows) {
+                    ck[cpos] = keys[j];
+                    ci[cpos] = p[j].x;
                 }
+                ++cpos;
             }
         }
+        win_base += tot & 0xffffu;
+        cand_base += tot >> 16;
     }
     __syncthreads();
     if (reinit) {
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
             state[unit].surv_cnt = 0;
         }
     }
-    uint32_t n_c = s_cand;
+    uint32_t n_c = cand_base;
     if (n_c > (uint32_t)n_rows) n_c = n_rows;
     if (c_less >= kk) return;
     uint32_t need = kk - c_less;

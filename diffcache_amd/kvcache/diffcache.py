@@ -100,6 +100,7 @@ class DiffCache:
                     for _ in range(num_layers)]
         self._ws: Optional[torch.Tensor] = None
         self._ws_rows = -1
+        self._ws_ready = False   # True once a decode_attention call has left the select state ready
         self._attn_out: Optional[torch.Tensor] = None
         self._prefix0 = kvbuf_prefix_len
         self._suffix0 = kvbuf_suffix_len
@@ -120,6 +121,7 @@ class DiffCache:
                 hip.layer_workspace_bytes(n_units, region, self.retrieval_budget, self.group,
                                           self.head_dim, attended), self.device)
             self._ws_rows = region
+            self._ws_ready = False
         return self._ws
 
     # ------------------------------------------------------------------ prefill
@@ -188,6 +190,7 @@ class DiffCache:
             ws = self._ensure_workspace()
             hip.score_select(self.kstore[layer_idx], self.qbuf, lo, hi - lo, retrieval_len, self.mode,
                              hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
+            self._ws_ready = False   # the one-shot call does not leave the state initialised
         assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
@@ -230,7 +233,8 @@ class DiffCache:
         ws = self._ensure_workspace()
         hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
                          self.kvbuf_suffix_len + 1, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
-                         mode=self.mode, order=order)
+                         mode=self.mode, order=order, select_state_ready=self._ws_ready)
+        self._ws_ready = True
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
         return out

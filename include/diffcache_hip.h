@@ -219,6 +219,13 @@ typedef struct dc_layer_args {
     int budget;           /* k */
     int mode, order;
     float scale;          /* softmax scale, 1/sqrt(hd) in the reference */
+    int select_state_ready; /* streaming select only (scores == NULL).  0: the workspace is
+                             initialised first.  1: the caller vouches that the last call on this
+                             workspace was a dc_decode_layer with the same n_b, n_h, region length
+                             and budget and scores == NULL, which leaves the select state ready;
+                             the init kernel is skipped */
+    void *ev_scan_begin;  /* optional hipEvent_t pair recorded on `stream` right before and */
+    void *ev_scan_end;    /* right after the scan kernel (for timing it in place), or NULL */
 } dc_layer_args;
 
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,
