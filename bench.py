@@ -185,14 +185,18 @@ def main() -> int:
             self.stream = torch.cuda.Stream(device=dev)     # default priority
             self.clean = False
 
-        def layer(self, l, ev=None):
+        def layer(self, l, ev=None, wait_for=None):
             k, v, q, nk, nv = self.layers[l]
             nu = self.n_units
+            if wait_for is not None:
+                # scans of different micro-batches take turns: this layer call starts once the
+                # other micro-batch's scan has finished, so its select/attention overlap our scan
+                torch.cuda.current_stream().wait_event(wait_for)
             if args.fused:
                 hip.decode_layer(q, k, v, sink, hi, recent, budget, self.scores, self.idx, self.out,
                                  self.ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY,
                                  select_state_ready=self.clean and not args.dense,
-                                 scan_events=None if ev is None or l % args.event_stride else
+                                 scan_events=None if ev is None or l % stride else
                                  (ev[4 * l], ev[4 * l + 1]))
                 self.clean = True
                 return
@@ -227,29 +231,35 @@ def main() -> int:
     def new_events(count):
         return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
 
-    def step(evs=None):
+    stride = 1 if args.streams > 1 else args.event_stride
+
+    def step(evs):
         """One decode step: every layer in order; the micro-batches are independent of
-        each other and each runs its layers in order on its own stream."""
+        each other and each runs its layers in order on its own stream.  With several
+        streams the scans are chained through their end events so that only one scan
+        streams from HBM at a time."""
+        prev_scan_end = None
         for l in range(L):
             for pi, pipe in enumerate(pipes):
                 with torch.cuda.stream(pipe.stream):
-                    pipe.layer(l, None if evs is None else evs[pi])
+                    pipe.layer(l, evs[pi], wait_for=prev_scan_end if args.streams > 1 else None)
+                if args.streams > 1:
+                    prev_scan_end = evs[pi][4 * l + 1]
 
-    for _ in range(args.warmup):
-        step()
+    events = [[new_events(4 * L) for _ in pipes] for _ in range(args.steps + 1)]
+    # torch creates the native event on first record; the C side needs the handle
+    for per_step in events:
+        for pi, evs in enumerate(per_step):
+            for e in evs:
+                e.record(pipes[pi].stream)
     torch.cuda.synchronize()
-    events = [[new_events(4 * L) for _ in pipes] for _ in range(args.steps)]
-    if args.fused:
-        # torch creates the native event on first record; the C side needs the handle
-        for per_step in events:
-            for pi, evs in enumerate(per_step):
-                for l in range(0, L, args.event_stride):
-                    evs[4 * l].record(pipes[pi].stream)
-                    evs[4 * l + 1].record(pipes[pi].stream)
-        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step(events[-1])
+    torch.cuda.synchronize()
+    events = events[:-1]
     t0 = time.perf_counter()
     for s in range(args.steps):
-        step(None if events is None else events[s])
+        step(events[s])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
@@ -259,7 +269,7 @@ def main() -> int:
     score_ms = None
     flat = [e for per_step in events for e in per_step]
     if args.fused:
-        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(0, L, args.event_stride)]
+        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(0, L, stride)]
         score_ms = sum(sc) / len(sc)
         stage_us = {"score": score_ms * 1e3, "timed_launches": len(sc)}
     else:

@@ -33,15 +33,14 @@ constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 4096;
 
-// tb_run is polled by every wave of the scan while ticket / surv_cnt take
-// returning atomics; they sit in separate 128-byte lines because polling a
-// line that is being updated atomically serialises both at the memory side.
+// tb_run is polled by every wave of the scan while surv_cnt takes returning
+// atomics; they sit in separate 128-byte lines because polling a line that is
+// being updated atomically serialises both at the memory side.
 struct UnitState {
     uint32_t tb_run;    // running threshold bucket (only decreases)
     uint32_t pad0[31];
-    uint32_t ticket;    // blocks of this unit that have flushed their histogram
     uint32_t surv_cnt;  // survivors appended so far
-    uint32_t pad1[30];
+    uint32_t pad1[31];
 };
 
 __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units) {
@@ -50,7 +49,6 @@ __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units)
     if (i < n_hist) hist[i] = 0;
     if (i < n_units) {
         state[i].tb_run = DC_HIST_BINS;  // nothing is pruned until a threshold exists
-        state[i].ticket = 0;
         state[i].surv_cnt = 0;
     }
 }
@@ -70,7 +68,8 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     __shared__ uint32_t lhist[DC_HIST_BINS];
     __shared__ uint2 stage[kStage];
     __shared__ uint32_t wtot[kThreads / 64 + 1];
-    __shared__ uint32_t s_cnt, s_base, s_ticket;
+    __shared__ uint32_t s_wcnt[kThreads / 64];
+    __shared__ uint32_t s_base;
 
     const int unit = blockIdx.x % n_units;
     const int chunk = blockIdx.x / n_units;
@@ -80,28 +79,37 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     const int grp = lane / LPR, col = lane % LPR;
 
     const bool small = chunk < small_chunks;
+    // Units sit a power of two apart in memory; rotating each unit's order of large
+    // chunks keeps blocks that run together from walking the same address offsets.
+    const int big_chunks = (int)(gridDim.x / n_units) - small_chunks;
+    const int big_id = small ? 0 : (int)(((int64_t)(chunk - small_chunks) + (int64_t)unit * 7) % big_chunks);
     const int64_t block_row0 =
         small ? (int64_t)chunk * kRowsPerBlockStep
-              : (int64_t)small_chunks * kRowsPerBlockStep +
-                    (int64_t)(chunk - small_chunks) * big_steps * kRowsPerBlockStep;
+              : (int64_t)small_chunks * kRowsPerBlockStep + (int64_t)big_id * big_steps * kRowsPerBlockStep;
     const int steps = small ? 1 : big_steps;
 
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
-    if (tid == 0) s_cnt = 0;
+
+    const uint16_t *Ku = K + b * sb + h * sh + col * 8;
+    UnitState *st = state + unit;
+    const int last = n_rows - 1;
+    uint32_t tb = load_relaxed(&st->tb_run);
 
     float q[8];
     dc_load_query<HD>(Q, unit, q_group, col, q);
     __syncthreads();
 
-    const uint16_t *Ku = K + b * sb + h * sh + col * 8;
-    UnitState *st = state + unit;
-    const int last = n_rows - 1;
+    // Each wave stages its survivors in its own slice of `stage` (at most 64 per
+    // step), so the cursor is a wave-uniform register and no LDS atomic is needed.
+    uint2 *wstage = stage + wave * (kBigSteps * 64);
+    uint32_t wcnt = 0;
+    const unsigned long long lt = (1ull << lane) - 1ull;
 
     for (int step = 0; step < steps; ++step) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
         if (row0 >= n_rows) break;  // wave-uniform; no barrier inside the loop
-        const uint32_t tb = load_relaxed(&st->tb_run);
         float mine = 0.f;
+        uint32_t tb_next = tb;
 #pragma unroll
         for (int c0 = 0; c0 < LPR; c0 += CH) {
             uint4 w[CH];
@@ -111,6 +119,8 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
                 r = r > last ? last : r;
                 w[j] = *reinterpret_cast<const uint4 *>(Ku + r * sr);
             }
+            // the threshold for the next step queues up behind this step's rows
+            if (c0 + CH >= LPR && step + 1 < steps) tb_next = load_relaxed(&st->tb_run);
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
                 float p = dc_group_sum<LPR>(dc_dot8(w[j], q, 0.f));
@@ -126,39 +136,36 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
         const bool keep = valid && bucket <= tb;
         if (keep) atomicAdd(&lhist[bucket], 1u);
         const unsigned long long mask = __ballot(keep);
-        if (mask) {
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(&s_cnt, (uint32_t)__popcll(mask));
-            base = __shfl(base, 0, 64);
-            if (keep) {
-                const uint32_t pos = base + __popcll(mask & ((1ull << lane) - 1ull));
-                stage[pos] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
-            }
-        }
+        if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+        wcnt += (uint32_t)__popcll(mask);
+        tb = tb_next;
     }
+    if (lane == 0) s_wcnt[wave] = wcnt;
     __syncthreads();
 
-    // append this block's survivors to the unit's list
-    const uint32_t cnt = s_cnt;
-    if (tid == 0) s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
-    __syncthreads();
-    {
-        uint2 *dst = surv + (int64_t)unit * n_rows + s_base;
-        for (uint32_t i = tid; i < cnt; i += kThreads) dst[i] = stage[i];
+    // append this block's survivors to the unit's list: one returning atomic per
+    // block, in flight while the histogram is flushed
+    uint32_t wbase = 0, cnt = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+        if (w2 < wave) wbase += s_wcnt[w2];
+        cnt += s_wcnt[w2];
     }
-    // add the block's histogram to the unit's
+    if (tid == 0) s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
     uint32_t *hu = hist + (int64_t)unit * DC_HIST_BINS;
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
         const uint32_t c = lhist[i];
         if (c) atomicAdd(&hu[i], c);
     }
     __syncthreads();
-    if (tid == 0) s_ticket = atomicAdd(&st->ticket, 1u);
-    __syncthreads();
-    // A few blocks per unit refresh the running threshold: every 4th of the
-    // first 32 to finish, then every 8th.  Staleness only loosens the bound.
-    const uint32_t ticket = s_ticket;
-    const bool refresh = ticket < 32u ? (ticket & 3u) == 3u : (ticket & 7u) == 7u;
+    {
+        uint2 *dst = surv + (int64_t)unit * n_rows + s_base + wbase;
+        for (uint32_t i = lane; i < wcnt; i += 64) dst[i] = wstage[i];
+    }
+    // A few blocks per unit refresh the running threshold from whatever part of
+    // the histogram is visible: every 4th small block, every 8th large one.
+    // Staleness only loosens the bound.
+    const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     if (!refresh) return;
 
     // Coalesced, L2-bypassing read of the unit's histogram into LDS (lhist is
@@ -304,7 +311,6 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
         hz[tid] = make_uint4(0u, 0u, 0u, 0u);
         if (tid == 0) {
             state[unit].tb_run = DC_HIST_BINS;
-            state[unit].ticket = 0;
             state[unit].surv_cnt = 0;
         }
     }
