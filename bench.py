@@ -26,6 +26,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one scan launch of the default workload moves, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE scaled by a known-size copy kernel (the figures and commands are kept with the
+# other profile summaries of this repository): 2.2103 GB read + 13.07 MB written.
+SCAN_TRAFFIC_BYTES_C3 = 2_223_300_000
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
@@ -127,6 +131,9 @@ def main() -> int:
                     help="pipeline the batch as this many independent micro-batches, one HIP stream each "
                          "(the units of a layer are independent, so one micro-batch's select/attention "
                          "overlaps the other's scan)")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="before the steps, run a plain elementwise kernel that reads 1 GiB and writes "
+                         "1 GiB three times (a known-size reference for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
@@ -246,6 +253,14 @@ def main() -> int:
                 if args.streams > 1:
                     prev_scan_end = evs[pi][4 * l + 1]
 
+    if args.pmc_calibration:
+        ca = torch.ones((256 << 20,), dtype=torch.float32, device=dev)      # 1 GiB
+        cb = torch.empty_like(ca)
+        for _ in range(3):
+            torch.add(ca, 1.0, out=cb)
+        torch.cuda.synchronize()
+        del ca, cb
+
     events = [[new_events(4 * L) for _ in pipes] for _ in range(args.steps + 1)]
     # torch creates the native event on first record; the C side needs the handle
     for per_step in events:
@@ -287,6 +302,8 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
                 "traffic": None, "kernel": "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
                 "algorithmic_bytes_per_launch": score_bytes}
+    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist":
+        roofline["traffic"] = SCAN_TRAFFIC_BYTES_C3
     if score_ms is not None:
         ach = score_bytes / (score_ms * 1e-3) / 1e9
         roofline.update(achieved=ach, frac=ach / HBM_PEAK_GBPS, avg_launch_us=score_ms * 1e3)

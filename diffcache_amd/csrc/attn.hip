@@ -37,7 +37,9 @@ struct AttnPlan {
 AttnPlan plan_attn(int hd, int n_units, int n_total) {
     AttnPlan p;
     const int batch = (kThreads / (hd / 8)) * kRowsPerGroup;
-    int target_splits = (1024 + n_units - 1) / (n_units > 0 ? n_units : 1);
+    // measured on MI355X: single-batch blocks (many small ones) beat longer pipelined blocks
+    // until the grid gets very large, so aim high
+    int target_splits = (4096 + n_units - 1) / (n_units > 0 ? n_units : 1);
     if (target_splits < 1) target_splits = 1;
     int iters = n_total > 0 ? (n_total + batch * target_splits - 1) / (batch * target_splits) : 1;
     if (iters < 1) iters = 1;
@@ -372,7 +374,7 @@ extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_
     // plan_attn never makes more than max(target_splits, ceil(n / (8 * batch))) splits for any
     // list of at most n rows, so a workspace sized for the longest list serves shorter ones
     const int batch = (kThreads / (hd / 8)) * kRowsPerGroup;
-    const int target = (1024 + n_units - 1) / n_units;
+    const int target = (4096 + n_units - 1) / n_units;
     const int by_cap = (n_rows_attended + kMaxIters * batch - 1) / (kMaxIters * batch);
     const int worst = target > by_cap ? target : (by_cap > 1 ? by_cap : 1);
     return carve_attn(nullptr, n_units, group, hd, worst).bytes;
