@@ -1,0 +1,95 @@
+"""PQ baseline on the HBM store: codebook training, encoding and the search
+pipeline ADC scan -> candidates -> exact bf16 rerank.
+
+The reference's PQ baseline directory (evaluation/impl/pqcache) is empty, so
+this follows the benchmark configuration only: M subspaces x 256 centroids,
+8-bit codes, per-query fp32 lookup tables, 4096 candidates reranked to top-k.
+Training and encoding are one-off preparation and use torch ops on the device;
+everything a query touches runs in libdiffcache_hip.so.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _hip as hip
+
+
+def train_codebooks(keys: torch.Tensor, m: int, iters: int = 8, seed: int = 0,
+                    n_centroids: int = 256) -> torch.Tensor:
+    """Seeded Lloyd k-means per subspace.  keys (n, hd) on the GPU ->
+    (m, n_centroids, hd/m) fp32.  Initial centroids are a seeded sample of the
+    keys; an empty cell keeps its centroid."""
+    x = keys.float()
+    n, hd = x.shape
+    ds = hd // m
+    g = torch.Generator(device=x.device).manual_seed(seed)
+    books = torch.empty((m, n_centroids, ds), dtype=torch.float32, device=x.device)
+    for j in range(m):
+        xs = x[:, j * ds:(j + 1) * ds].contiguous()
+        c = xs[torch.randint(0, n, (n_centroids,), generator=g, device=x.device)].clone()
+        for _ in range(iters):
+            a = torch.cdist(xs, c).argmin(dim=1)
+            sums = torch.zeros_like(c).index_add_(0, a, xs)
+            cnt = torch.bincount(a, minlength=n_centroids).to(xs.dtype)
+            nz = cnt > 0
+            c[nz] = sums[nz] / cnt[nz, None]
+        books[j] = c
+    return books
+
+
+def encode(keys: torch.Tensor, books: torch.Tensor, chunk: int = 1 << 18) -> torch.Tensor:
+    """keys (n, hd) bf16/fp32, books (m, 256, ds) -> codes (n, m) uint8: nearest
+    centroid by squared L2 per subspace."""
+    m, nc, ds = books.shape
+    n = keys.shape[0]
+    codes = torch.empty((n, m), dtype=torch.uint8, device=keys.device)
+    for s in range(0, n, chunk):
+        x = keys[s:s + chunk].float()
+        for j in range(m):
+            d = torch.cdist(x[:, j * ds:(j + 1) * ds].contiguous(), books[j])
+            codes[s:s + chunk, j] = d.argmin(dim=1).to(torch.uint8)
+    return codes
+
+
+class PQIndex:
+    """Codes and codebooks of every (batch, kv-head) unit over an HBM key store
+    (bsz, kv_heads, n, hd); codebooks are shared by the batch elements of a head."""
+
+    def __init__(self, store_k: torch.Tensor, books: torch.Tensor, codes: torch.Tensor,
+                 n_cand: int = 4096, topk: int = 1024) -> None:
+        b, h, n, hd = store_k.shape
+        assert books.shape[0] == h and books.shape[2] == 256 and books.dtype == torch.float32
+        assert codes.shape == (b * h, n, books.shape[1]) and codes.dtype == torch.uint8
+        self.store_k, self.books, self.codes = store_k, books.contiguous(), codes.contiguous()
+        self.b, self.h, self.n, self.hd, self.m = b, h, n, hd, books.shape[1]
+        self.n_cand, self.topk = min(n_cand, n), min(topk, n)
+        dev = store_k.device
+        nu = b * h
+        self.hist = hip.new_hist(nu, dev)
+        self.cand = torch.empty((nu, self.n_cand), dtype=torch.int32, device=dev)
+        self.pos = torch.empty((nu, self.topk), dtype=torch.int32, device=dev)
+        self.ws1 = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, n, self.n_cand), dev)
+        self.ws2 = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, self.n_cand, self.topk), dev)
+
+    @classmethod
+    def build(cls, store_k: torch.Tensor, m: int = 32, sample: int = 65536, iters: int = 8,
+              seed: int = 0, **kw) -> "PQIndex":
+        b, h, n, hd = store_k.shape
+        books = torch.stack([train_codebooks(store_k[0, hh, :min(sample, n)], m, iters, seed + hh)
+                             for hh in range(h)])
+        codes = torch.stack([encode(store_k[bb, hh], books[hh]) for bb in range(b) for hh in range(h)])
+        return cls(store_k, books, codes, **kw)
+
+    def search(self, q: torch.Tensor) -> torch.Tensor:
+        """q (b*h, hd) bf16 -> int32 ids (b*h, topk), best exact score first."""
+        lut = hip.pq_build_lut(q, self.books, self.b)
+        self.hist.zero_()
+        adc = hip.pq_adc_scan(self.codes, lut, hist=self.hist)
+        cand = hip.topk_select(adc, self.n_cand, hip.MODE_IP, hip.ORDER_INDEX, hist=self.hist,
+                               idx_out=self.cand, workspace=self.ws1)
+        exact = hip.score_gathered(self.store_k, q, cand)
+        pos = hip.topk_select(exact, self.topk, hip.MODE_IP, hip.ORDER_BEST, idx_out=self.pos,
+                              workspace=self.ws2)
+        return hip.compose_idx(cand, pos)

@@ -290,3 +290,38 @@ def test_diffcache_prefill_cache_roundtrip(tmp_path):
         n_att = c.seq_len_gpu(1) - 0
         outs.append(np_u16(c.get_kvcache(1)[0])[:, :budget + p + s])
     assert np.array_equal(outs[0], outs[1])
+
+
+# ---------------------------------------------------------------- PQ baseline
+
+def test_pq_index_search_matches_oracle_pipeline():
+    """PQIndex.search = ADC scan -> candidates -> exact rerank; codes and tables are
+    checked against the numpy oracle, ids against the oracle's pipeline run on the
+    GPU's own ADC and exact scores."""
+    from diffcache_amd import _hip
+    from diffcache_amd.pq import PQIndex, encode, train_codebooks
+    rng = np.random.default_rng(50)
+    b, h, n, hd, m = 1, 2, 30000, 128, 32
+    keys = rand_bf16(rng, b, h, n, hd)
+    store = dev_bf16(keys)
+    index = PQIndex.build(store, m=m, sample=8192, iters=3, seed=1, n_cand=1024, topk=128)
+    books = index.books.cpu().numpy()
+    codes = index.codes.cpu().numpy()
+    for u in range(h):
+        want = orc.pq_encode(orc.bf16_to_f32(keys[0, u]), books[u])
+        # the nearest centroid may tie within fp32 rounding of the distance: allow a handful
+        assert np.mean(codes[u] != want) < 1e-3
+    q = rand_bf16(rng, h, hd)
+    ids = index.search(dev_bf16(q)).cpu().numpy()
+    lut = _hip.pq_build_lut(dev_bf16(q), index.books, b).cpu().numpy()
+    adc = _hip.pq_adc_scan(index.codes, torch.from_numpy(lut).to(DEV)).cpu().numpy()
+    for u in range(h):
+        assert np.allclose(lut[u], orc.pq_build_lut(q[u], books[u]), rtol=1e-5, atol=1e-5)
+        assert np.allclose(adc[u], orc.pq_adc_scores(codes[u], lut[u].astype(np.float64)), rtol=1e-5, atol=1e-4)
+        cand = np.sort(orc.topk_select(adc[u], 1024, orc.MODE_IP))
+        exact = _hip.score_gathered(store, dev_bf16(q), torch.from_numpy(
+            np.stack([cand, cand]).astype(np.int32)).to(DEV)).cpu().numpy()[u]
+        order = orc.topk_select(exact, 128, orc.MODE_IP)
+        assert np.array_equal(ids[u], cand[order])
+        true = set(orc.topk_select(orc.scores_f32(q[u], keys[0, u]), 128, orc.MODE_IP).tolist())
+        assert len(true & set(ids[u].tolist())) >= 40      # recall of ADC with 1024 candidates
