@@ -3,15 +3,15 @@
 // call of src/diffcache/base.py:134-142: the selected rows are read straight
 // from the HBM-resident store instead of being copied into a dense buffer.
 //
-// Grid: one block per (unit, split); a split is a slice of kRowsPerGroup * NG
+// Grid: one block per (unit, split); a split is a slice of rows_per_group * NG
 // consecutive positions of the unit's attended list [selected | sinks | recent |
-// current token] walked in batches of 64 rows (at head_dim 128).  A group of
-// LPR = HD/8 lanes owns one row at a time (one 16-byte load per lane covers the
-// row) and the G query heads of the GQA group share every row that is loaded.
-// The K and V rows of the next batch are requested while the current batch is
-// reduced; logits stay in registers and every row group keeps its own running
-// (m, l, acc), merged over the block at the end.  Each split leaves (m, l, acc)
-// in the workspace; merge_kernel combines the splits through their log-sum-exp.  (Merging in the last block to arrive was tried:
+// current token] (128 rows at head_dim 128 and a GQA group of 4).  A group of LPR = HD/8 lanes owns one
+// row at a time (one 16-byte load per lane covers the row) and the G query heads
+// of the GQA group share every row that is loaded.  All K and V rows of the
+// slice are requested up front (one memory round trip after the id lookup), the
+// logits stay in registers, the block agrees on a per-head maximum, and each
+// split leaves (m, l, acc) in the workspace; merge_kernel combines the splits
+// through their log-sum-exp.  (Merging in the last block to arrive was tried:
 // the device-scope fence it needs costs far more than a second launch here.)
 // Bound by HBM: 2 * HD*2 bytes per row.
 #include "dc_common.h"
@@ -21,31 +21,19 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
-constexpr int kRowsPerGroup = 4;
-constexpr int kMaxIters = 8;
+// rows a lane group takes per block: 8 while the GQA group is small, 4 when the per-head
+// registers (queries, logits, accumulators) leave less room
+__host__ __device__ constexpr int rows_per_group(int group) { return group <= 4 ? 8 : 4; }
 constexpr uint32_t kNewToken = 0xffffffffu;
 
 struct AttnPlan {
-    int iters;           // row batches a block walks through
-    int rows_per_split;  // NG * kRowsPerGroup * iters
+    int rows_per_split;
     int n_splits;
 };
 
-// Splits are sized so that a layer gives a few hundred blocks: fewer, longer
-// blocks keep several loads in flight per lane (the next batch of rows is
-// requested while the current one is reduced) and leave fewer partials to merge.
-AttnPlan plan_attn(int hd, int n_units, int n_total) {
+AttnPlan plan_attn(int hd, int group, int n_total) {
     AttnPlan p;
-    const int batch = (kThreads / (hd / 8)) * kRowsPerGroup;
-    // measured on MI355X: single-batch blocks (many small ones) beat longer pipelined blocks
-    // until the grid gets very large, so aim high
-    int target_splits = (4096 + n_units - 1) / (n_units > 0 ? n_units : 1);
-    if (target_splits < 1) target_splits = 1;
-    int iters = n_total > 0 ? (n_total + batch * target_splits - 1) / (batch * target_splits) : 1;
-    if (iters < 1) iters = 1;
-    if (iters > kMaxIters) iters = kMaxIters;
-    p.iters = iters;
-    p.rows_per_split = batch * iters;
+    p.rows_per_split = (kThreads / (hd / 8)) * rows_per_group(group);
     p.n_splits = n_total > 0 ? (n_total + p.rows_per_split - 1) / p.rows_per_split : 1;
     return p;
 }
@@ -56,24 +44,39 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const uint32_t *__restrict__ idx, const uint16_t *__restrict__ new_k,
     const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml, int n_h,
     int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-    int n_total, int n_splits, int iters, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
-    int64_t vsh, int64_t vsr, float scale) {
+    int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
+    int64_t vsr, float scale) {
     constexpr int LPR = HD / 8;
     constexpr int NG = kThreads / LPR;  // row groups per block
-    constexpr int R = kRowsPerGroup;
-    constexpr int GPW = 64 / LPR;       // groups per wave
-    __shared__ float s_m[kWaves][G];
+    constexpr int R = rows_per_group(G);
+    constexpr int ROWS = NG * R;
+    __shared__ float s_red[kWaves][G];
     __shared__ float s_l[kWaves][G];
     __shared__ float s_acc[kWaves][G * HD];
-    __shared__ uint32_t s_rows[NG * R * kMaxIters];
 
     const int unit = blockIdx.x / n_splits;
     const int split = blockIdx.x % n_splits;
     const int b = unit / n_h, h = unit % n_h;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gid = tid / LPR, col = tid % LPR;
-    const int r0 = split * (NG * R * iters);
+    const int r0 = split * ROWS;
 
+    // physical rows of this group's list positions
+    uint32_t row[R];
+    bool ok[R];
+#pragma unroll
+    for (int t = 0; t < R; ++t) {
+        const int vj = r0 + t * NG + gid;
+        ok[t] = vj < n_total;
+        uint32_t r = 0;
+        if (ok[t]) {
+            if (vj < n_idx) r = (uint32_t)(region_lo + idx[(int64_t)unit * idx_stride + vj]);
+            else if (vj < n_idx + n_sink) r = (uint32_t)(vj - n_idx);
+            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
+            else r = kNewToken;
+        }
+        row[t] = r;
+    }
     float qf[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -91,154 +94,110 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const uint16_t *Vu = V + b * vsb + h * vsh + col * 8;
     const uint16_t *nk = new_k ? new_k + (int64_t)unit * HD + col * 8 : Ku;
     const uint16_t *nv = new_v ? new_v + (int64_t)unit * HD + col * 8 : Vu;
-    const uint32_t *iu = idx + (int64_t)unit * idx_stride;
 
-    // physical row of every list position of the split, staged in LDS with one
-    // coalesced read of the ids (kNewToken = the current token's own k/v)
-    for (int j = tid; j < NG * R * iters; j += kThreads) {
-        const int vj = r0 + j;
-        uint32_t r = 0u;
-        if (vj < n_total) {
-            if (vj < n_idx) r = (uint32_t)(region_lo + iu[vj]);
-            else if (vj < n_idx + n_sink) r = (uint32_t)(vj - n_idx);
-            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
-            else r = kNewToken;
-        }
-        s_rows[j] = r;
+    // every K and V row of the slice is requested before any is used
+    uint4 kw[R], vw[R];
+#pragma unroll
+    for (int t = 0; t < R; ++t) {
+        const uint16_t *pk = (row[t] == kNewToken) ? nk : Ku + (int64_t)row[t] * ksr;
+        kw[t] = *reinterpret_cast<const uint4 *>(pk);
     }
-    __syncthreads();
-    auto load_batch = [&](int it, uint4 (&kw)[R], uint4 (&vw)[R]) {
-        uint32_t row[R];
 #pragma unroll
-        for (int t = 0; t < R; ++t) row[t] = s_rows[(it * R + t) * NG + gid];
-#pragma unroll
-        for (int t = 0; t < R; ++t)
-            kw[t] = *reinterpret_cast<const uint4 *>((row[t] == kNewToken) ? nk : Ku + (int64_t)row[t] * ksr);
-#pragma unroll
-        for (int t = 0; t < R; ++t)
-            vw[t] = *reinterpret_cast<const uint4 *>((row[t] == kNewToken) ? nv : Vu + (int64_t)row[t] * vsr);
-    };
+    for (int t = 0; t < R; ++t) {
+        const uint16_t *pv = (row[t] == kNewToken) ? nv : Vu + (int64_t)row[t] * vsr;
+        vw[t] = *reinterpret_cast<const uint4 *>(pv);
+    }
 
-    // running (m, l, acc) of this row group; all lanes of the group agree on m and l
-    float m[G], l[G], acc[G][8];
+    // scaled logits, in registers: x[t][g] is known to every lane of the group
+    float x[R][G];
+    float mloc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) mloc[g] = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < R; ++t)
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float v = dc_group_sum<LPR>(dc_dot8(kw[t], qf[g], 0.f)) * scale;
+            x[t][g] = ok[t] ? v : -INFINITY;
+            mloc[g] = fmaxf(mloc[g], x[t][g]);
+        }
+    // per-head maximum over the block
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        m[g] = -INFINITY;
-        l[g] = 0.f;
+        float v = mloc[g];
+#pragma unroll
+        for (int off = LPR; off < 64; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+        if (lane == 0) s_red[wave][g] = v;
+    }
+    __syncthreads();
+    float m[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float v = s_red[0][g];
+#pragma unroll
+        for (int w2 = 1; w2 < kWaves; ++w2) v = fmaxf(v, s_red[w2][g]);
+        m[g] = v;
+    }
+
+    // p = exp(x - m), acc[g] += p * V
+    float acc[G][8];
+    float lloc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        lloc[g] = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
     }
-
-    uint4 kw[R], vw[R], kn[R], vn[R];
-    load_batch(0, kw, vw);
-    for (int it = 0; it < iters; ++it) {
-        if (it + 1 < iters) load_batch(it + 1, kn, vn);  // in flight while this batch is reduced
-        float x[R][G];
-        float mb[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) mb[g] = m[g];
-#pragma unroll
-        for (int t = 0; t < R; ++t) {
-            const bool ok = r0 + (it * R + t) * NG + gid < n_total;
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const float v = dc_group_sum<LPR>(dc_dot8(kw[t], qf[g], 0.f)) * scale;
-                x[t][g] = ok ? v : -INFINITY;
-                mb[g] = fmaxf(mb[g], x[t][g]);
-            }
-        }
+    for (int t = 0; t < R; ++t) {
+        const float v[8] = {dc_bf16_lo(vw[t].x), dc_bf16_hi(vw[t].x), dc_bf16_lo(vw[t].y),
+                            dc_bf16_hi(vw[t].y), dc_bf16_lo(vw[t].z), dc_bf16_hi(vw[t].z),
+                            dc_bf16_lo(vw[t].w), dc_bf16_hi(vw[t].w)};
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const float corr = (m[g] > -INFINITY) ? __expf(m[g] - mb[g]) : 0.f;
-            l[g] *= corr;
+            const float p = ok[t] ? __expf(x[t][g] - m[g]) : 0.f;
+            lloc[g] += p;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] *= corr;
-            m[g] = mb[g];
-        }
-#pragma unroll
-        for (int t = 0; t < R; ++t) {
-            const float v[8] = {dc_bf16_lo(vw[t].x), dc_bf16_hi(vw[t].x), dc_bf16_lo(vw[t].y),
-                                dc_bf16_hi(vw[t].y), dc_bf16_lo(vw[t].z), dc_bf16_hi(vw[t].z),
-                                dc_bf16_lo(vw[t].w), dc_bf16_hi(vw[t].w)};
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const float p = (x[t][g] > -INFINITY) ? __expf(x[t][g] - m[g]) : 0.f;
-                l[g] += p;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
-            }
-        }
-        if (it + 1 < iters) {
-#pragma unroll
-            for (int t = 0; t < R; ++t) {
-                kw[t] = kn[t];
-                vw[t] = vn[t];
-            }
+            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
         }
     }
 
-    // merge the row groups of a wave: common maximum, rescale, add
+    // reduce over the row groups: inside the wave, then across waves
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float mw = m[g];
+    for (int off = LPR; off < 64; off <<= 1)
 #pragma unroll
-        for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
-        const float corr = (m[g] > -INFINITY) ? __expf(m[g] - mw) : 0.f;
-        l[g] *= corr;
+        for (int g = 0; g < G; ++g) {
+            lloc[g] += __shfl_xor(lloc[g], off, 64);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] *= corr;
-        m[g] = mw;
-    }
-    if (GPW > 1) {
-#pragma unroll
-        for (int off = LPR; off < 64; off <<= 1)
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                l[g] += __shfl_xor(l[g], off, 64);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g][i] += __shfl_xor(acc[g][i], off, 64);
-            }
-    }
+            for (int i = 0; i < 8; ++i) acc[g][i] += __shfl_xor(acc[g][i], off, 64);
+        }
     if (lane < LPR) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            if (col == 0) {
-                s_m[wave][g] = m[g];
-                s_l[wave][g] = l[g];
-            }
+            if (col == 0) s_l[wave][g] = lloc[g];
 #pragma unroll
             for (int i = 0; i < 8; ++i) s_acc[wave][g * HD + col * 8 + i] = acc[g][i];
         }
     }
     __syncthreads();
-    // merge the waves and leave the split's partial result
     const int64_t slot = (int64_t)unit * n_splits + split;
     for (int o = tid; o < G * HD; o += kThreads) {
-        const int g = o / HD;
-        float mm = s_m[0][g];
+        float s = s_acc[0][o];
 #pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) mm = fmaxf(mm, s_m[w2][g]);
-        float s = 0.f;
-#pragma unroll
-        for (int w2 = 0; w2 < kWaves; ++w2) {
-            const float mw = s_m[w2][g];
-            if (mw > -INFINITY) s += __expf(mw - mm) * s_acc[w2][o];
-        }
+        for (int w2 = 1; w2 < kWaves; ++w2) s += s_acc[w2][o];
         ws_acc[slot * (G * HD) + o] = s;
     }
     if (tid < G) {
-        float mm = s_m[0][tid];
+        float l = s_l[0][tid];
 #pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) mm = fmaxf(mm, s_m[w2][tid]);
-        float ll = 0.f;
+        for (int w2 = 1; w2 < kWaves; ++w2) l += s_l[w2][tid];
+        float mm = s_red[0][tid];
 #pragma unroll
-        for (int w2 = 0; w2 < kWaves; ++w2) {
-            const float mw = s_m[w2][tid];
-            if (mw > -INFINITY) ll += __expf(mw - mm) * s_l[w2][tid];
-        }
+        for (int w2 = 1; w2 < kWaves; ++w2) mm = fmaxf(mm, s_red[w2][tid]);
         ws_ml[(slot * G + tid) * 2 + 0] = mm;
-        ws_ml[(slot * G + tid) * 2 + 1] = ll;
+        ws_ml[(slot * G + tid) * 2 + 1] = l;
     }
+
 }
 
 // out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block
@@ -344,14 +303,14 @@ int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const u
                 const uint16_t *v, const uint32_t *idx, const uint16_t *new_k,
                 const uint16_t *new_v, const AttnWs &w, int n_h, int n_idx,
                 int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-                int n_total, int n_splits, int iters, int64_t ksb, int64_t ksh, int64_t ksr,
-                int64_t vsb, int64_t vsh, int64_t vsr, float scale) {
+                int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
+                int64_t vsh, int64_t vsr, float scale) {
 #define DC_ATTN_CASE(GG)                                                                           \
     case GG:                                                                                       \
         hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, q, k, v, idx, \
                            new_k, new_v, w.acc, w.ml, n_h, n_idx, idx_stride,                      \
-                           region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, iters, ksb,  \
-                           ksh, ksr, vsb, vsh, vsr, scale);                                        \
+                           region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, ksb, ksh,    \
+                           ksr, vsb, vsh, vsr, scale);                                             \
         return 0;
     switch (group) {
         DC_ATTN_CASE(1)
@@ -371,13 +330,7 @@ int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const u
 
 extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attended) {
     if (n_units <= 0 || group <= 0 || hd < 8) return 256;
-    // plan_attn never makes more than max(target_splits, ceil(n / (8 * batch))) splits for any
-    // list of at most n rows, so a workspace sized for the longest list serves shorter ones
-    const int batch = (kThreads / (hd / 8)) * kRowsPerGroup;
-    const int target = (4096 + n_units - 1) / n_units;
-    const int by_cap = (n_rows_attended + kMaxIters * batch - 1) / (kMaxIters * batch);
-    const int worst = target > by_cap ? target : (by_cap > 1 ? by_cap : 1);
-    return carve_attn(nullptr, n_units, group, hd, worst).bytes;
+    return carve_attn(nullptr, n_units, group, hd, plan_attn(hd, group, n_rows_attended).n_splits).bytes;
 }
 
 extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
@@ -409,7 +362,7 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
     const int n_total = n_idx + n_sink + n_recent + (new_k ? 1 : 0);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "dc_gather_attn_bf16: workspace must be non-null and 256-byte aligned");
-    const AttnPlan plan = plan_attn(hd, n_units, n_total);
+    const AttnPlan plan = plan_attn(hd, group, n_total);
     const AttnWs w = carve_attn(workspace, n_units, group, hd, plan.n_splits);
     if (workspace_bytes < w.bytes) {
         dc_set_error("dc_gather_attn_bf16: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
@@ -425,15 +378,15 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
     if (hd == 64)
         rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                             plan.n_splits, plan.iters, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+                             plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else if (hd == 128)
         rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan.n_splits, plan.iters, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else
         rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan.n_splits, plan.iters, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     DC_REQUIRE(rc == 0, "dc_gather_attn_bf16: unsupported group %d", group);
     DC_CHECK_LAUNCH("dc_gather_attn_bf16(attn)");
     hipLaunchKernelGGL(merge_kernel, dim3((unsigned)(n_units * group)), dim3(hd), 0, st, w.acc, w.ml, o16,
