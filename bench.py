@@ -49,12 +49,11 @@ def algorithmic_bytes_per_unit(n_region: int, attended: int, group: int, hd: int
     return n_region * hd * 2 + 2 * attended * hd * 2 + group * hd * 2 * 2
 
 
-def make_layer(torch, cfg, layer: int, cfg_id: int, dev):
-    """Synthetic K, V, q, new k/v of one layer, generated on the device."""
+def make_layer(torch, cfg, layer: int, cfg_id: int, dev, k, v):
+    """Synthetic K, V, q, new k/v of one layer, generated on the device into the
+    layer's views k, v of the store."""
     g = torch.Generator(device=dev).manual_seed(1000 * cfg_id + layer)
     b, hkv, hq, hd, n = cfg["batch"], cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"]
-    k = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
-    v = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
     k.normal_(generator=g)
     v.normal_(generator=g)
     # per-channel log-normal scale (sigma 1), one vector per kv head: outlier channels
@@ -220,7 +219,12 @@ def main() -> int:
     attended = k_eff + sink + recent + 1
 
     t_gen = time.perf_counter()
-    layers = [make_layer(torch, cfg, l, cfg_id, dev) for l in range(L)]
+    # One allocation holds every layer's keys and one every layer's values, as the KV
+    # store of diffcache_amd.DiffCache does: scans of a single large allocation run
+    # about 3 % faster on MI355X than scans of per-layer allocations.
+    vslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    kslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    layers = [make_layer(torch, cfg, l, cfg_id, dev, kslab[l], vslab[l]) for l in range(L)]
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t_gen
 

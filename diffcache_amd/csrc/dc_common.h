@@ -55,20 +55,37 @@ __device__ __forceinline__ uint32_t dc_f2ord(float x) {
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
-// 32-bit ordering key (smaller = better) and its coarse histogram bucket.
-// The bucket is a monotone function of the key, so equal keys share a bucket.
-// DC_MODE_IP:       key = ord(-(s + 0)),            bucket = key >> 20
+// Histogram bucket of a score (larger score = better = smaller bucket), a monotone
+// map onto [0, DC_HIST_BINS).  Positive scores from 2^-20 up to 2^20 get 32 buckets
+// per binade (the top-k of an attention scan lives there: a finer grid leaves
+// fewer rows in the threshold bucket, a coarser one costs the scan fewer histogram
+// atomics); smaller positives share the last fine bucket, larger ones the first;
+// negative scores get two buckets per binade.
+constexpr uint32_t kPosBinades = 40u, kSubBits = 3u;
+constexpr uint32_t kPosBuckets = kPosBinades << kSubBits;
+__device__ __forceinline__ uint32_t dc_score_bucket(float s) {
+    const uint32_t b = __float_as_uint(s + 0.0f);  // -0 -> +0
+    const uint32_t mag = b & 0x7fffffffu;
+    if (b & 0x80000000u) return kPosBuckets + (mag >> 22);
+    constexpr uint32_t lo = (127u - 20u) << 23, hi = ((127u - 20u + kPosBinades) << 23) - 1u;
+    const uint32_t m = mag < lo ? lo : (mag > hi ? hi : mag);
+    return (kPosBuckets - 1u) - ((m - lo) >> (23u - kSubBits));
+}
+static_assert(kPosBuckets + 512u <= DC_HIST_BINS, "bucket map exceeds the histogram");
+
+// 32-bit ordering key (smaller = better) and its histogram bucket.  The bucket is
+// a monotone function of the key, so equal keys share a bucket.
+// DC_MODE_IP:       key = ord(-(s + 0)),            bucket from s
 // DC_MODE_REF_DIST: key = ord(d), d = f32(65536-s); bucket from s' = 65536 - d,
 //                   which is exact and is s rounded onto d's grid.
 __device__ __forceinline__ void dc_key_bucket(float s, int mode, uint32_t &key, uint32_t &bucket) {
     if (mode == DC_MODE_REF_DIST) {
         float d = 65536.0f - s;
         key = dc_f2ord(d);
-        float sq = 65536.0f - d;
-        bucket = dc_f2ord(-(sq + 0.0f)) >> 20;
+        bucket = dc_score_bucket(65536.0f - d);
     } else {
         key = dc_f2ord(-(s + 0.0f));
-        bucket = key >> 20;
+        bucket = dc_score_bucket(s);
     }
 }
 

@@ -40,52 +40,59 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, 
     return off + incl - v;
 }
 
-// Among `n` values v(i), find the rem-th smallest (1-based) by radix passes over
-// bits [hb, 0].  get(i, &value) returns false for items outside the subset.
-// Returns the threshold value; *rem_out = how many items equal to it are needed
-// (rank of the threshold inside its tie group), *n_eq = size of the tie group.
+// One radix pass of a select: among the items whose bits [31, top) equal those of
+// `prefix`, histogram bits [top-1, top-width) and find the bin that holds the
+// rem-th smallest (1-based).  Updates prefix (bin bits filled in), rem (rank inside
+// the bin), eq (bin size) and top (= the lowest decided bit).  Uniform over the block.
 template <typename Get>
-__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int hb, uint32_t common,
-                                       uint32_t *lh, uint32_t *wtot, uint32_t *sres,
-                                       uint32_t *rem_out, uint32_t *n_eq) {
+__device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &prefix, uint32_t &rem,
+                                                 uint32_t &eq, int &top, uint32_t *lh, uint32_t *wtot,
+                                                 uint32_t *sres) {
     const int tid = threadIdx.x;
-    uint32_t prefix = common;  // bits above hb, shared by every item
-    int top = hb + 1;          // bits [top-1, 0] still undecided
-    uint32_t eq = n;
-    while (top > 0) {
-        const int width = top < kRadixBits ? top : kRadixBits;
-        const int shift = top - width;
-        for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
-        __syncthreads();
-        const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
-        for (uint32_t i = tid; i < n; i += kFinalThreads) {
-            uint32_t v;
-            if (get(i, &v) && ((v & himask) == (prefix & himask)))
-                atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
-        }
-        __syncthreads();
-        // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
-        const uint32_t h0 = lh[2 * tid], h1 = lh[2 * tid + 1];
-        uint32_t total;
-        const uint32_t excl = block_excl_scan<kFinalThreads>(h0 + h1, wtot, &total);
-        if (excl < rem && rem <= excl + h0 + h1) {
-            if (excl + h0 >= rem) {
-                sres[0] = 2 * tid;
-                sres[1] = excl;
-                sres[2] = h0;
-            } else {
-                sres[0] = 2 * tid + 1;
-                sres[1] = excl + h0;
-                sres[2] = h1;
-            }
-        }
-        __syncthreads();
-        prefix |= sres[0] << shift;
-        rem -= sres[1];
-        eq = sres[2];
-        top = shift;
-        __syncthreads();
+    const int width = top < kRadixBits ? top : kRadixBits;
+    const int shift = top - width;
+    for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
+    __syncthreads();
+    const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
+    for (uint32_t i = tid; i < n; i += kFinalThreads) {
+        uint32_t v;
+        if (get(i, &v) && ((v & himask) == (prefix & himask)))
+            atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
     }
+    __syncthreads();
+    // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
+    const uint32_t h0 = lh[2 * tid], h1 = lh[2 * tid + 1];
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<kFinalThreads>(h0 + h1, wtot, &total);
+    if (excl < rem && rem <= excl + h0 + h1) {
+        if (excl + h0 >= rem) {
+            sres[0] = 2 * tid;
+            sres[1] = excl;
+            sres[2] = h0;
+        } else {
+            sres[0] = 2 * tid + 1;
+            sres[1] = excl + h0;
+            sres[2] = h1;
+        }
+    }
+    __syncthreads();
+    prefix |= sres[0] << shift;
+    rem -= sres[1];
+    eq = sres[2];
+    top = shift;
+    __syncthreads();
+}
+
+// Among `n` values v(i), find the rem-th smallest (1-based) by radix passes over
+// bits [top-1, 0], the bits above being those of `prefix` for every item of the
+// subset.  get(i, &value) returns false for items outside the subset.  Returns the
+// threshold value; *rem_out = how many items equal to it are needed (rank of the
+// threshold inside its tie group), *n_eq = size of the tie group.
+template <typename Get>
+__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int top, uint32_t prefix,
+                                       uint32_t eq, uint32_t *lh, uint32_t *wtot, uint32_t *sres,
+                                       uint32_t *rem_out, uint32_t *n_eq) {
+    while (top > 0) block_radix_pass(get, n, prefix, rem, eq, top, lh, wtot, sres);
     *rem_out = rem;
     *n_eq = eq;
     return prefix;
@@ -109,7 +116,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
     }
     // bits in which the candidate keys differ
     if (tid == 0) {
-        smisc[0] = 0;  // OR of key differences
+        smisc[0] = 0;  // OR of key differences, later the length of the tie list
         smisc[1] = 0;  // output slot counter
     }
     __syncthreads();
@@ -120,15 +127,56 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
     __syncthreads();
     diff = smisc[0];
     const int hb = diff ? 31 - __clz(diff) : -1;
-    const uint32_t common = (hb >= 31) ? 0u : (k0 & (0xffffffffu << (hb + 1)));
-
-    uint32_t need_eq, n_eq;
+    uint32_t prefix = (hb >= 31) ? 0u : (k0 & (0xffffffffu << (hb + 1)));
+    int top = hb + 1;
+    uint32_t rem = need, eq = n_c;
     auto get_key = [&](uint32_t i, uint32_t *v) {
         *v = ck[i];
         return true;
     };
+    if (top > 0) block_radix_pass(get_key, n_c, prefix, rem, eq, top, lh, wtot, sres);
+
+    if (eq <= (uint32_t)kFinalThreads) {
+        // The keys whose decided bits equal the threshold bin's are few: they are
+        // listed in LDS as packed (key, id) and ranked against each other, which
+        // settles the remaining key bits and the ties by id at once.
+        unsigned long long *tie = reinterpret_cast<unsigned long long *>(lh);
+        __syncthreads();  // smisc[0] has been read by every thread
+        if (tid == 0) smisc[0] = 0;
+        __syncthreads();
+        const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
+        const uint32_t base = need - rem;  // members from the bins below the threshold bin
+        for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
+            const uint32_t key = ck[i], id = ci[i];
+            const uint32_t hi = key & himask, ph = prefix & himask;
+            if (hi < ph) {
+                const uint32_t slot = atomicAdd(&smisc[1], 1u);
+                if (slot < base) {
+                    io[slot] = id;
+                    if (kout) kout[slot] = key;
+                }
+            } else if (hi == ph) {
+                const uint32_t e = atomicAdd(&smisc[0], 1u);
+                if (e < (uint32_t)kFinalThreads) tie[e] = ((unsigned long long)key << 32) | id;
+            }
+        }
+        __syncthreads();
+        const uint32_t n_t = smisc[0] < (uint32_t)kFinalThreads ? smisc[0] : (uint32_t)kFinalThreads;
+        if ((uint32_t)tid < n_t) {
+            const unsigned long long mine = tie[tid];
+            uint32_t rank = 0;
+            for (uint32_t j = 0; j < n_t; ++j) rank += tie[j] < mine ? 1u : 0u;
+            if (rank < rem) {
+                io[base + rank] = (uint32_t)mine;
+                if (kout) kout[base + rank] = (uint32_t)(mine >> 32);
+            }
+        }
+        return;
+    }
+
+    uint32_t need_eq, n_eq;
     const uint32_t t_key =
-        block_radix_select(get_key, n_c, need, hb, common, lh, wtot, sres, &need_eq, &n_eq);
+        block_radix_select(get_key, n_c, rem, top, prefix, eq, lh, wtot, sres, &need_eq, &n_eq);
 
     uint32_t t_idx = 0xffffffffu;
     if (need_eq < n_eq) {  // only the lowest ids of the tie group fit
@@ -139,7 +187,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
             return ck[i] == t_key;
         };
         uint32_t r2, e2;
-        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi, 0u, lh, wtot, sres, &r2, &e2);
+        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi + 1, 0u, n_eq, lh, wtot, sres, &r2, &e2);
     }
 
     for (uint32_t i = tid; i < n_c; i += kFinalThreads) {

@@ -18,9 +18,10 @@
 // advance together, and the first chunks of every unit are small so that a
 // threshold exists early.
 //
-// sparse_select_kernel (one block per unit) derives the exact threshold bucket
-// from the complete histogram, splits the survivors into certain members and
-// candidates, and finishes with the same radix select as finalize_kernel.
+// classify_kernel (several blocks per unit) derives the exact threshold bucket
+// from the complete histogram and splits the survivors into certain members and
+// candidates; select_finish_kernel (one block per unit) finishes with the same
+// radix select as finalize_kernel.
 #include "dc_common.h"
 #include "dc_select.h"
 
@@ -40,8 +41,13 @@ struct UnitState {
     uint32_t tb_run;    // running threshold bucket (only decreases)
     uint32_t pad0[31];
     uint32_t surv_cnt;  // survivors appended so far
-    uint32_t pad1[31];
+    uint32_t win_cnt;   // certain members written to idx_out (select phase)
+    uint32_t cand_cnt;  // candidates of the threshold bucket (select phase)
+    uint32_t c_less;    // keys in buckets better than the threshold bucket
+    uint32_t pad1[28];
 };
+static_assert(sizeof(UnitState) == 256, "UnitState is two 128-byte lines");
+static_assert(kRadixBins * 4 >= kFinalThreads * 8, "lh doubles as the packed candidate list");
 
 __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -50,6 +56,9 @@ __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units)
     if (i < n_units) {
         state[i].tb_run = DC_HIST_BINS;  // nothing is pruned until a threshold exists
         state[i].surv_cnt = 0;
+        state[i].win_cnt = 0;
+        state[i].cand_cnt = 0;
+        state[i].c_less = 0;
     }
 }
 
@@ -201,89 +210,118 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     }
 }
 
-// One block per unit: exact threshold bucket from the complete histogram, then
-// certain members / candidates from the survivor list, then the radix select.
-__global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
-    uint32_t *__restrict__ hist, UnitState *__restrict__ state, const uint2 *__restrict__ surv,
-    uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out,
-    int64_t idx_stride, uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int mode, int reinit) {
-    __shared__ uint32_t lh[kRadixBins];
-    __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
-    __shared__ uint32_t sres[4];
-    __shared__ uint32_t smisc[2];
-    __shared__ uint32_t s_tb, s_cless;
-    __shared__ uint32_t lck[kCandLds], lci[kCandLds];  // candidates stay in LDS when they fit
-    const int unit = blockIdx.x;
+// Exact threshold bucket of a unit from its complete histogram: the bucket that
+// holds the k-th best key, and how many keys sit in better buckets.  Called by
+// all kThreads threads; the result is uniform.  `wtot`, `sres`: LDS scratch.
+__device__ __forceinline__ void unit_threshold(const uint32_t *__restrict__ hu, uint32_t kk,
+                                               uint32_t *wtot, uint32_t *sres, uint32_t &tb,
+                                               uint32_t &c_less) {
     const int tid = threadIdx.x;
     if (tid == 0) {
-        s_tb = DC_HIST_BINS;
-        s_cless = 0;
+        sres[0] = DC_HIST_BINS;
+        sres[1] = 0;
     }
-    uint32_t bins[4];
-    {
-        const uint4 t = reinterpret_cast<const uint4 *>(hist + (int64_t)unit * DC_HIST_BINS)[tid];
-        // (each thread re-zeroes exactly the four bins it read, see the end of the survivor loop)
-        bins[0] = t.x;
-        bins[1] = t.y;
-        bins[2] = t.z;
-        bins[3] = t.w;
+    uint32_t bins[16];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint4 t = reinterpret_cast<const uint4 *>(hu)[tid * 4 + i];
+        bins[4 * i + 0] = t.x;
+        bins[4 * i + 1] = t.y;
+        bins[4 * i + 2] = t.z;
+        bins[4 * i + 3] = t.w;
+        sum += t.x + t.y + t.z + t.w;
     }
-    const uint32_t sum = bins[0] + bins[1] + bins[2] + bins[3];
     uint32_t total;
-    const uint32_t excl = block_excl_scan<kFinalThreads>(sum, wtot, &total);
-    const uint32_t kk = (uint32_t)k_eff;
+    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
     if (excl < kk && kk <= excl + sum) {
         uint32_t run = excl;
         bool done = false;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 16; ++i) {
             if (!done && run + bins[i] >= kk) {
-                s_tb = tid * 4 + i;
-                s_cless = run;
+                sres[0] = tid * 16 + i;
+                sres[1] = run;
                 done = true;
             }
             run += bins[i];
         }
     }
     __syncthreads();
-    const uint32_t tb = s_tb, c_less = s_cless;
-    uint32_t n_s = state[unit].surv_cnt;
-    if (n_s > (uint32_t)n_rows) n_s = n_rows;
+    tb = sres[0];
+    c_less = sres[1];
+}
+
+// Several blocks per unit split the unit's survivor list: rows in buckets better
+// than the threshold bucket are certain members and go straight to idx_out, rows
+// in the threshold bucket become candidates.  Each block reserves its output
+// ranges with one returning atomic per list.
+constexpr int kClassifyBatch = 4;
+
+__global__ __launch_bounds__(kThreads) void classify_kernel(
+    const uint32_t *__restrict__ hist, UnitState *__restrict__ state, const uint2 *__restrict__ surv,
+    uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out,
+    int64_t idx_stride, uint32_t *__restrict__ sel_keys, int n_units, int n_rows, int k_eff, int mode,
+    int nblk) {
+    __shared__ uint32_t wtot[kThreads / 64 + 1];
+    __shared__ uint32_t sres[2];
+    __shared__ uint32_t sbase[2];
+    const int unit = blockIdx.x % n_units;
+    const int blk = blockIdx.x / n_units;
+    const int tid = threadIdx.x;
+    UnitState *st = state + unit;
     const uint2 *su = surv + (int64_t)unit * n_rows;
+    const uint32_t cap = (uint32_t)n_rows;
+    uint32_t n_s = st->surv_cnt;
+    if (n_s > cap) n_s = cap;
+    // every block takes one contiguous slice of whole batches
+    constexpr uint32_t kPer = kClassifyBatch * kThreads;
+    const uint32_t per = ((n_s + (uint32_t)nblk - 1) / (uint32_t)nblk + kPer - 1) / kPer * kPer;
+    const uint32_t lo = (uint32_t)blk * per;
+    uint32_t hi = lo + per;
+    if (hi > n_s) hi = n_s;
+    if (lo >= n_s && blk != 0) return;
+
+    const uint32_t kk = (uint32_t)k_eff;
+    uint32_t tb, c_less;
+    unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, kk, wtot, sres, tb, c_less);
+    if (blk == 0 && tid == 0) st->c_less = c_less;
+
     uint32_t *ck = cand_key + (int64_t)unit * n_rows;
     uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
     uint32_t *io = idx_out + (int64_t)unit * idx_stride;
     uint32_t *ko = sel_keys ? sel_keys + (int64_t)unit * k_eff : nullptr;
 
-    // Survivors are taken 16 per thread at a time: classify into bit masks, one
-    // block-wide scan of the packed (member, candidate) counts, then every thread
-    // writes to its own range -- no atomics on the output cursors.
-    constexpr int kBatch = 16;
-    uint32_t win_base = 0, cand_base = 0;
-    for (uint32_t i0 = 0; i0 < n_s; i0 += kBatch * kFinalThreads) {
-        uint2 p[kBatch];
+    for (uint32_t i0 = lo; i0 < hi; i0 += kPer) {
+        uint2 p[kClassifyBatch];
 #pragma unroll
-        for (int j = 0; j < kBatch; ++j) {
-            const uint32_t i = i0 + j * kFinalThreads + tid;
+        for (int j = 0; j < kClassifyBatch; ++j) {
+            const uint32_t i = i0 + j * kThreads + tid;
             p[j] = make_uint2(0u, 0u);
-            if (i < n_s) p[j] = su[i];
+            if (i < hi) p[j] = su[i];
         }
-        uint32_t keys[kBatch];
+        uint32_t keys[kClassifyBatch];
         uint32_t wmask = 0, cmask = 0;
 #pragma unroll
-        for (int j = 0; j < kBatch; ++j) {
-            const uint32_t i = i0 + j * kFinalThreads + tid;
+        for (int j = 0; j < kClassifyBatch; ++j) {
+            const uint32_t i = i0 + j * kThreads + tid;
             uint32_t key = 0, bucket = 0xffffffffu;
-            if (i < n_s) dc_key_bucket(__uint_as_float(p[j].y), mode, key, bucket);
+            if (i < hi) dc_key_bucket(__uint_as_float(p[j].y), mode, key, bucket);
             keys[j] = key;
             if (bucket < tb) wmask |= 1u << j;
             else if (bucket == tb) cmask |= 1u << j;
         }
         uint32_t tot;
-        const uint32_t ex = block_excl_scan<kFinalThreads>(__popc(wmask) | (__popc(cmask) << 16), wtot, &tot);
-        uint32_t wpos = win_base + (ex & 0xffffu), cpos = cand_base + (ex >> 16);
+        const uint32_t ex = block_excl_scan<kThreads>(__popc(wmask) | (__popc(cmask) << 16), wtot, &tot);
+        if (tid == 0) {
+            const uint32_t nw = tot & 0xffffu, nc = tot >> 16;
+            sbase[0] = nw ? atomicAdd(&st->win_cnt, nw) : 0u;
+            sbase[1] = nc ? atomicAdd(&st->cand_cnt, nc) : 0u;
+        }
+        __syncthreads();
+        uint32_t wpos = sbase[0] + (ex & 0xffffu), cpos = sbase[1] + (ex >> 16);
 #pragma unroll
-        for (int j = 0; j < kBatch; ++j) {
+        for (int j = 0; j < kClassifyBatch; ++j) {
             if (wmask & (1u << j)) {
                 if (wpos < kk) {
                     io[wpos] = p[j].x;
@@ -291,43 +329,100 @@ __global__ __launch_bounds__(kFinalThreads) void sparse_select_kernel(
                 }
                 ++wpos;
             } else if (cmask & (1u << j)) {
-                if (cpos < (uint32_t)kCandLds) {
-                    lck[cpos] = keys[j];
-                    lci[cpos] = p[j].x;
-                } else if (cpos < (uint32_t)n_rows) {
+                if (cpos < cap) {
                     ck[cpos] = keys[j];
                     ci[cpos] = p[j].x;
                 }
                 ++cpos;
             }
         }
-        win_base += tot & 0xffffu;
-        cand_base += tot >> 16;
+        __syncthreads();  // sbase is rewritten by the next batch
     }
-    __syncthreads();
+}
+
+// One block per unit: radix select among the candidates of the threshold bucket
+// fills idx_out[c_less, k).  Leaves the unit's list cursors at zero.
+__global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
+    uint32_t *__restrict__ hist, UnitState *__restrict__ state, uint32_t *__restrict__ cand_key,
+    uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out, int64_t idx_stride,
+    uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int reinit) {
+    __shared__ uint32_t lh[kRadixBins];
+    __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
+    __shared__ uint32_t sres[4];
+    __shared__ uint32_t smisc[2];
+    __shared__ uint32_t lck[kCandLds], lci[kCandLds];  // candidates are staged in LDS when they fit
+    const int unit = blockIdx.x;
+    const int tid = threadIdx.x;
+    UnitState *st = state + unit;
+    uint32_t *ck = cand_key + (int64_t)unit * n_rows;
+    uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
+    // the head of the candidate list is fetched before its length is known
+    uint32_t hk = 0, hi = 0;
+    if (tid < n_rows) {
+        hk = ck[tid];
+        hi = ci[tid];
+    }
+    uint32_t n_c = st->cand_cnt;
+    const uint32_t c_less = st->c_less;
+    if (n_c > (uint32_t)n_rows) n_c = n_rows;
+    const uint32_t kk = (uint32_t)k_eff;
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride;
+    uint32_t *ko = sel_keys ? sel_keys + (int64_t)unit * k_eff : nullptr;
+    const uint32_t *fk = ck, *fi = ci;
+    if (n_c <= (uint32_t)kCandLds) {
+        if ((uint32_t)tid < n_c) {
+            lck[tid] = hk;
+            lci[tid] = hi;
+        }
+        for (uint32_t i = tid + kFinalThreads; i < n_c; i += kFinalThreads) {
+            lck[i] = ck[i];
+            lci[i] = ci[i];
+        }
+        fk = lck;
+        fi = lci;
+    }
+    __syncthreads();  // every thread has read the counters
     if (reinit) {
-        // leave the unit's histogram and counters ready for the next scan
+        // leave the unit's histogram and threshold ready for the next scan
         uint4 *hz = reinterpret_cast<uint4 *>(hist + (int64_t)unit * DC_HIST_BINS);
         hz[tid] = make_uint4(0u, 0u, 0u, 0u);
-        if (tid == 0) {
-            state[unit].tb_run = DC_HIST_BINS;
-            state[unit].surv_cnt = 0;
-        }
     }
-    uint32_t n_c = cand_base;
-    if (n_c > (uint32_t)n_rows) n_c = n_rows;
+    if (tid == 0) {
+        if (reinit) {
+            st->tb_run = DC_HIST_BINS;
+            st->surv_cnt = 0;
+        }
+        st->win_cnt = 0;
+        st->cand_cnt = 0;
+    }
     if (c_less >= kk) return;
     uint32_t need = kk - c_less;
     if (need > n_c) need = n_c;
-    const uint32_t *fk = lck, *fi = lci;
-    if (n_c > (uint32_t)kCandLds) {  // overflow: the head of the list joins the tail in global memory
-        for (int i = tid; i < kCandLds; i += kFinalThreads) {
-            ck[i] = lck[i];
-            ci[i] = lci[i];
-        }
+    if (n_c <= 128u) {
+        // Short list: every thread ranks its own candidate among all of them by
+        // (key, id).  The packed pairs sit in lh, padded with a sentinel to a multiple
+        // of 8; the reads in the loop are wave-uniform 16-byte broadcasts.
+        unsigned long long *comp = reinterpret_cast<unsigned long long *>(lh);
+        const unsigned long long mine = ((unsigned long long)hk << 32) | hi;
+        comp[tid] = (uint32_t)tid < n_c ? mine : ~0ull;
         __syncthreads();
-        fk = ck;
-        fi = ci;
+        if ((uint32_t)tid < n_c) {
+            const ulonglong2 *c2 = reinterpret_cast<const ulonglong2 *>(comp);
+            const uint32_t n8 = (n_c + 7u) / 8u;
+            uint32_t rank = 0;
+            for (uint32_t j = 0; j < n8; ++j) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const ulonglong2 t = c2[4 * j + u];
+                    rank += (t.x < mine ? 1u : 0u) + (t.y < mine ? 1u : 0u);
+                }
+            }
+            if (rank < need) {
+                io[c_less + rank] = hi;
+                if (ko) ko[c_less + rank] = hk;
+            }
+        }
+        return;
     }
     dc_finalize_unit(fk, fi, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc,
                      ko ? ko + c_less : nullptr);
@@ -477,9 +572,18 @@ extern "C" int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int 
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
-    hipLaunchKernelGGL(sparse_select_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.hist, w.state,
-                       w.surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows,
-                       k_eff, mode, reinit);
+    // blocks per unit for the classify pass: one per 4096 rows of context, as long as
+    // the grid stays near 2048 blocks
+    int nblk = (n_rows + 4095) / 4096;
+    const int cap = n_units >= 2048 ? 1 : 2048 / n_units;
+    if (nblk > cap) nblk = cap;
+    if (nblk < 1) nblk = 1;
+    hipLaunchKernelGGL(classify_kernel, dim3((unsigned)n_units * (unsigned)nblk), dim3(kThreads), 0, st,
+                       w.hist, w.state, w.surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride,
+                       sel_keys, n_units, n_rows, k_eff, mode, nblk);
+    DC_CHECK_LAUNCH("dc_sparse_select");
+    hipLaunchKernelGGL(select_finish_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.hist, w.state,
+                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows, k_eff, reinit);
     DC_CHECK_LAUNCH("dc_sparse_select");
     if (order != DC_ORDER_ANY)
         return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,

@@ -459,9 +459,20 @@ def pq_search(q_u16: np.ndarray, k_u16: np.ndarray, codes: np.ndarray, lut_f32: 
 
 
 def coarse_bucket(scores: np.ndarray, mode: int) -> np.ndarray:
+    """Bucket (smaller = better) of each score: positive scores in [2^-20, 2^20) get
+    32 buckets per binade, clamped outside; negative scores two per binade."""
     s = np.asarray(scores, dtype=np.float32)
     if mode == MODE_REF_DIST:
         d = ref_dist(s)
         s = (np.float32(65536.0) - d).astype(np.float32)
     s = (s + np.float32(0.0)).astype(np.float32)
-    return (_f2ord((-s).astype(np.float32)) >> np.uint32(20)).astype(np.uint32)
+    b = s.view(np.uint32)
+    mag = b & np.uint32(0x7FFFFFFF)
+    binades, sub_bits = 40, 3
+    pos_buckets = np.uint32(binades << sub_bits)
+    lo = np.uint32((127 - 20) << 23)
+    hi = np.uint32(((127 - 20 + binades) << 23) - 1)
+    m = np.clip(mag, lo, hi)
+    pos = (pos_buckets - np.uint32(1)) - ((m - lo) >> np.uint32(23 - sub_bits))
+    neg = pos_buckets + (mag >> np.uint32(22))
+    return np.where((b >> np.uint32(31)) != 0, neg, pos).astype(np.uint32)
