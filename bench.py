@@ -28,8 +28,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one scan launch of the default workload moves, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a known-size copy kernel (the figures and commands are kept with the
-# other profile summaries of this repository): 2.2103 GB read + 13.07 MB written.
-SCAN_TRAFFIC_BYTES_C3 = 2_223_300_000
+# other profile summaries of this repository): 1 053 933 counts x 2 KiB read +
+# 12 570 counts x 1 KiB written.
+SCAN_TRAFFIC_BYTES_C3 = 1_053_933 * 2048 + 12_570 * 1024
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
