@@ -191,7 +191,13 @@ def main() -> int:
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
+    ap.add_argument("--sketch", action="store_true",
+                    help="scan the 8-bit sketch of the keys and rescore the surviving rows exactly "
+                         "(dc_score_select_sketch_bf16 inside dc_decode_layer): same ids, half the bytes")
     args = ap.parse_args()
+    if args.sketch and (args.dense or args.split or args.streams != 1):
+        print("bench.py: --sketch goes with the default one-call path only", file=sys.stderr)
+        return 2
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
               "use --gpus 1", file=sys.stderr)
@@ -226,6 +232,11 @@ def main() -> int:
     vslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
     kslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
     layers = [make_layer(torch, cfg, l, cfg_id, dev, kslab[l], vslab[l]) for l in range(L)]
+    sketches = None
+    if args.sketch:
+        # the sketch of the retrieval region of every layer (prefill-time work, untimed)
+        cslab = torch.empty((L, b, hkv, n, hd), dtype=torch.uint8, device=dev)
+        sketches = [hip.Sketch(kslab[l], codes=cslab[l]).build(kslab[l], lo, hi - lo) for l in range(L)]
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t_gen
 
@@ -265,7 +276,8 @@ def main() -> int:
                                  self.ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY,
                                  select_state_ready=self.clean and not args.dense,
                                  scan_events=None if ev is None or l % stride else
-                                 (ev[4 * l], ev[4 * l + 1]))
+                                 (ev[4 * l], ev[4 * l + 1]),
+                                 sketch=None if sketches is None else sketches[l])
                 self.clean = True
                 return
             if args.dense:
@@ -359,11 +371,15 @@ def main() -> int:
     unit_bytes = algorithmic_bytes_per_unit(region, k_eff + sink + recent, grp, hd)
     step_bytes = unit_bytes * n_units * L
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
-    score_bytes = (n_units // args.streams) * region * hd * 2   # K rows streamed by one scan launch
+    # bytes one scan launch has to stream: the bf16 K rows, or their one-byte-per-element sketch
+    score_bytes = (n_units // args.streams) * region * hd * (1 if args.sketch else 2)
     roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
-                "traffic": None, "kernel": "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
+                "traffic": None,
+                "kernel": "sketch_prune_kernel<128>" if args.sketch else
+                          "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
                 "algorithmic_bytes_per_launch": score_bytes}
-    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist":
+    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist" \
+            and not args.sketch:
         roofline["traffic"] = SCAN_TRAFFIC_BYTES_C3
     if score_ms is not None:
         ach = score_bytes / (score_ms * 1e-3) / 1e9
@@ -383,7 +399,9 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": cfg["desc"], "key_mode": args.mode, "streams": args.streams,
-                   "call_path": ("dc_decode_layer" + (" (dense scores)" if args.dense else "") if args.fused else
+                   "call_path": ("dc_decode_layer" + (" (dense scores)" if args.dense else
+                                                      " (sketch scan + exact rescoring)" if args.sketch else "")
+                                 if args.fused else
                                  "dc_score_bf16/dc_topk_select/dc_gather_attn_bf16" if args.dense else
                                  "dc_select_state_init/dc_score_prune_bf16/dc_sparse_select/dc_gather_attn_bf16")},
         "step_hbm_gbps": step_gbps,

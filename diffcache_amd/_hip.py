@@ -32,6 +32,8 @@ SYMBOLS = (
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
     "dc_sparse_select", "dc_score_select_bf16",
+    "dc_sketch_build_bf16", "dc_sketch_select_workspace_bytes", "dc_sketch_select_state_init",
+    "dc_score_select_sketch_bf16",
 )
 
 
@@ -50,6 +52,9 @@ class LayerArgs(C.Structure):
         ("mode", C.c_int), ("order", C.c_int), ("scale", C.c_float),
         ("select_state_ready", C.c_int),
         ("ev_scan_begin", C.c_void_p), ("ev_scan_end", C.c_void_p),
+        ("sketch_codes", C.c_void_p), ("sketch_scale", C.c_void_p), ("sketch_resid", C.c_void_p),
+        ("sketch_batch_stride", C.c_int64), ("sketch_head_stride", C.c_int64),
+        ("sketch_row_stride", C.c_int64),
     ]
 
 
@@ -84,6 +89,11 @@ def _load() -> C.CDLL:
         "dc_score_prune_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i, i, i, p, sz, p]),
         "dc_sparse_select": (i, [p, i64, i, i, i, i, i, i, p, sz, p]),
         "dc_score_select_bf16": (i, [p, p, p, i64, i, i, i, i, i64, i64, i64, i, i, i, i, p, sz, p]),
+        "dc_sketch_build_bf16": (i, [p, p, p, p, i, i, i, i, i64, i64, i64, i64, i64, i64, i, p]),
+        "dc_sketch_select_workspace_bytes": (sz, [i, i, i]),
+        "dc_sketch_select_state_init": (i, [i, i, i, p, sz, p]),
+        "dc_score_select_sketch_bf16": (i, [p, p, p, p, p, p, i64, i, i, i, i, i64, i64, i64, i64, i64, i64,
+                                            i, i, i, i, i, p, sz, p, p, p]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -244,6 +254,66 @@ def score_select(store_k: torch.Tensor, q: torch.Tensor, lo: int, n_rows: int, b
     return idx_out[:, :k_eff]
 
 
+class Sketch:
+    """8-bit sketch of a (b, h, n, hd) bf16 key store: ``codes`` (b, h, n, hd) uint8 with
+    row r of the sketch describing row r of the store, ``scale`` and ``resid`` (b*h, hd)
+    fp32 (see dc_sketch_build_bf16 in the header)."""
+
+    def __init__(self, store_k: torch.Tensor, codes: Optional[torch.Tensor] = None):
+        _store_strides(store_k)
+        b, h, n, hd = store_k.shape
+        self.codes = torch.empty((b, h, n, hd), dtype=torch.uint8, device=store_k.device) \
+            if codes is None else codes
+        if self.codes.shape != store_k.shape or self.codes.dtype != torch.uint8 or self.codes.stride(3) != 1:
+            raise DiffCacheError("sketch codes must be a (b, h, n, hd) uint8 tensor with contiguous rows")
+        self.scale = torch.zeros((b * h, hd), dtype=torch.float32, device=store_k.device)
+        self.resid = torch.zeros((b * h, hd), dtype=torch.float32, device=store_k.device)
+
+    def build(self, store_k: torch.Tensor, lo: int, n_rows: int, keep_scale: bool = False) -> "Sketch":
+        """Sketch rows [lo, lo + n_rows).  keep_scale=False fits the scales to these rows
+        (prefill); keep_scale=True keeps them and only raises the residual bounds (append)."""
+        sb, sh, sr = _store_strides(store_k)
+        b, h, n_max, hd = store_k.shape
+        if lo < 0 or lo + n_rows > n_max:
+            raise DiffCacheError(f"rows [{lo}, {lo + n_rows}) outside the store of {n_max} rows")
+        c = self.codes
+        _check(lib.dc_sketch_build_bf16(
+            _dev(store_k, "store_k") + lo * sr * 2, _dev(c, "codes") + lo * c.stride(2),
+            _dev(self.scale, "scale"), _dev(self.resid, "resid"), b, h, n_rows, hd, sb, sh, sr,
+            c.stride(0), c.stride(1), c.stride(2), int(keep_scale), _stream()))
+        return self
+
+
+def sketch_select_workspace_bytes(n_units: int, n_rows: int, budget: int) -> int:
+    return int(lib.dc_sketch_select_workspace_bytes(n_units, n_rows, budget))
+
+
+def score_select_sketch(store_k: torch.Tensor, sketch: Sketch, q: torch.Tensor, lo: int, n_rows: int,
+                        budget: int, mode: int = MODE_REF_DIST, order: int = ORDER_ANY, q_group: int = 1,
+                        idx_out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                        state_ready: bool = False,
+                        scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None
+                        ) -> torch.Tensor:
+    """The ids of ``score_select`` (exact top-k of the bf16 keys), found by scanning the
+    8-bit sketch and rescoring the rows that can still matter."""
+    kptr, b, h, hd, sb, sh, sr = _score_select_args(store_k, q, lo, n_rows, q_group)
+    k_eff = min(budget, n_rows)
+    if idx_out is None:
+        idx_out = torch.empty((b * h, max(k_eff, 1)), dtype=torch.int32, device=store_k.device)
+    if workspace is None:
+        workspace = alloc_workspace(sketch_select_workspace_bytes(b * h, n_rows, budget), store_k.device)
+    c = sketch.codes
+    ev0 = ev1 = None
+    if scan_events is not None:
+        ev0, ev1 = scan_events[0].cuda_event, scan_events[1].cuda_event
+    _check(lib.dc_score_select_sketch_bf16(
+        kptr, _dev(c, "codes") + lo * c.stride(2), _dev(sketch.scale, "scale"), _dev(sketch.resid, "resid"),
+        _dev(q, "q"), _dev(idx_out, "idx_out"), idx_out.stride(0), b, h, n_rows, hd, sb, sh, sr,
+        c.stride(0), c.stride(1), c.stride(2), q_group, budget, mode, order, int(state_ready),
+        _dev(workspace, "workspace"), workspace.numel(), ev0, ev1, _stream()))
+    return idx_out[:, :k_eff]
+
+
 def gather_rows(store_k: Optional[torch.Tensor], store_v: Optional[torch.Tensor], idx: torch.Tensor,
                 out_k: Optional[torch.Tensor], out_v: Optional[torch.Tensor], row_offset: int = 0,
                 n_idx: Optional[int] = None) -> None:
@@ -332,9 +402,11 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
                  lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
                  order: int = ORDER_ANY, scale: Optional[float] = None,
                  select_state_ready: bool = False,
-                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None) -> torch.Tensor:
+                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
+                 sketch: Optional["Sketch"] = None) -> torch.Tensor:
     """score -> select -> attend for one layer, enqueued on the current stream.
-    ``select_state_ready``: see dc_layer_args in the header (skips the init kernel)."""
+    ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
+    ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result)."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
         raise DiffCacheError("K and V stores must share their strides")
@@ -362,6 +434,13 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
     if scan_events is not None:
         # torch creates the underlying event lazily: both must have been recorded once before
         a.ev_scan_begin, a.ev_scan_end = scan_events[0].cuda_event, scan_events[1].cuda_event
+    if sketch is not None:
+        c = sketch.codes
+        if c.shape != store_k.shape:
+            raise DiffCacheError("the sketch does not belong to this store")
+        a.sketch_codes, a.sketch_scale = _dev(c, "codes"), _dev(sketch.scale, "scale")
+        a.sketch_resid = _dev(sketch.resid, "resid")
+        a.sketch_batch_stride, a.sketch_head_stride, a.sketch_row_stride = c.stride(0), c.stride(1), c.stride(2)
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
 

@@ -40,9 +40,9 @@ LayerWs carve_layer(void *base, int n_units, int n_region, int budget, int group
     w.hist = (uint32_t *)(p + off);
     off += dc_align_up((size_t)(n_units > 0 ? n_units : 0) * DC_HIST_BINS * 4, 256);
     w.topk = p + off;
-    {   // room for either select path: dense scores + dc_topk_select, or the streaming one
+    {   // room for any select path: dense scores + dc_topk_select, or a streaming one
         size_t a = dc_topk_workspace_bytes(n_units, n_region, budget);
-        size_t b = dc_score_select_workspace_bytes(n_units, n_region, budget);
+        size_t b = dc_sketch_select_workspace_bytes(n_units, n_region, budget);
         w.topk_bytes = dc_align_up(a > b ? a : b, 256);
     }
     off += w.topk_bytes;
@@ -66,6 +66,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     DC_REQUIRE(a->n_b >= 0 && a->n_h >= 1 && a->group >= 1 && a->n_sink >= 0 && a->n_recent >= 0 &&
                    a->budget >= 0,
                "dc_decode_layer: bad sizes");
+    DC_REQUIRE(!(a->sketch_codes && a->scores), "dc_decode_layer: the sketch path needs scores == NULL");
     DC_REQUIRE(a->recent_lo >= a->n_sink, "dc_decode_layer: recent_lo %lld < n_sink %d",
                (long long)a->recent_lo, a->n_sink);
     const int n_units = a->n_b * a->n_h;
@@ -86,7 +87,17 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     int rc;
     const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
-    if (k_eff > 0 && !a->scores) {
+    if (k_eff > 0 && !a->scores && a->sketch_codes) {
+        // streaming select over the 8-bit sketch, exact rescoring of the kept rows
+        DC_REQUIRE(a->sketch_scale && a->sketch_resid, "dc_decode_layer: sketch_scale / sketch_resid missing");
+        rc = dc_score_select_sketch_bf16(
+            k_region, a->sketch_codes + (int64_t)a->n_sink * a->sketch_row_stride, a->sketch_scale,
+            a->sketch_resid, a->q, a->idx_out, a->idx_unit_stride, a->n_b, a->n_h, region, a->hd,
+            a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride, a->sketch_batch_stride,
+            a->sketch_head_stride, a->sketch_row_stride, a->group, a->budget, a->mode, a->order,
+            a->select_state_ready, w.topk, w.topk_bytes, a->ev_scan_begin, a->ev_scan_end, stream);
+        if (rc) return rc;
+    } else if (k_eff > 0 && !a->scores) {
         // no dense scores wanted: streaming score + select
         if (!a->select_state_ready) {
             rc = dc_select_state_init(n_units, region, a->budget, w.topk, w.topk_bytes, stream);

@@ -89,6 +89,19 @@ __device__ __forceinline__ void dc_key_bucket(float s, int mode, uint32_t &key, 
     }
 }
 
+// Margin of the sketch scan: a row can belong to the exact top-k only if
+// approx + margin reaches the k-th largest approx.  e = sum_d |q_d| r_d bounds the
+// quantisation error of one score, wabs = sum_d |q_d a_d| scales the fp32 rounding
+// of both the approximate and the exact evaluation (128-term dots of values up to
+// 127 a_d: below 1.5e-3 wabs together).  In DC_MODE_REF_DIST keys f32(65536 - s)
+// of unequal scores can tie, within one ulp of the key: 2^-23 (65536 + |s|).
+__device__ __forceinline__ float dc_sketch_margin(float e, float wabs, int mode) {
+    const float ep = 1.02f * e + 4.0e-3f * wabs;
+    float m = 2.0f * ep;
+    if (mode == DC_MODE_REF_DIST) m += (65536.0f + 128.0f * wabs + e) * 4.8e-7f;
+    return m;
+}
+
 // sum over the 16 lanes of a DPP row; every lane of the row receives the sum
 __device__ __forceinline__ float dc_row16_sum(float v) {
     v += __builtin_amdgcn_update_dpp(0.0f, v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]

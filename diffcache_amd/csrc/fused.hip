@@ -44,7 +44,8 @@ struct UnitState {
     uint32_t win_cnt;   // certain members written to idx_out (select phase)
     uint32_t cand_cnt;  // candidates of the threshold bucket (select phase)
     uint32_t c_less;    // keys in buckets better than the threshold bucket
-    uint32_t pad1[28];
+    uint32_t margin;    // sketch scan only: float bits of the score margin of the unit
+    uint32_t pad1[27];
 };
 static_assert(sizeof(UnitState) == 256, "UnitState is two 128-byte lines");
 static_assert(kRadixBins * 4 >= kFinalThreads * 8, "lh doubles as the packed candidate list");
@@ -59,11 +60,76 @@ __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units)
         state[i].win_cnt = 0;
         state[i].cand_cnt = 0;
         state[i].c_less = 0;
+        state[i].margin = 0;
     }
 }
 
 __device__ __forceinline__ uint32_t load_relaxed(const uint32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// End of a scan block: append the block's survivors (staged per wave in LDS) to
+// the unit's list with one returning atomic, flush the block's histogram, and in
+// the blocks chosen by the caller refresh the unit's running threshold from
+// whatever part of the histogram is visible.  Staleness only loosens the bound.
+__device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 *wstage, uint32_t wcnt,
+                                                   uint32_t *s_wcnt, uint32_t *s_base, uint32_t *wtot,
+                                                   UnitState *st, uint32_t *hu, uint2 *surv_unit,
+                                                   bool refresh, uint32_t kk) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    if (lane == 0) s_wcnt[wave] = wcnt;
+    __syncthreads();
+
+    // the atomic is in flight while the histogram is flushed
+    uint32_t wbase = 0, cnt = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+        if (w2 < wave) wbase += s_wcnt[w2];
+        cnt += s_wcnt[w2];
+    }
+    if (tid == 0) *s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
+        const uint32_t c = lhist[i];
+        if (c) atomicAdd(&hu[i], c);
+    }
+    __syncthreads();
+    {
+        uint2 *dst = surv_unit + *s_base + wbase;
+        for (uint32_t i = lane; i < wcnt; i += 64) dst[i] = wstage[i];
+    }
+    if (!refresh) return;
+
+    // Coalesced, L2-bypassing read of the unit's histogram into LDS (lhist is
+    // free again), then 16 adjacent bins per thread.
+    {
+        const unsigned long long *h64 = reinterpret_cast<const unsigned long long *>(hu);
+        unsigned long long *l64 = reinterpret_cast<unsigned long long *>(lhist);
+        for (int i = tid; i < DC_HIST_BINS / 2; i += kThreads)
+            l64[i] = __hip_atomic_load(h64 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    uint32_t bins[16];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        bins[i] = lhist[tid * 16 + i];
+        sum += bins[i];
+    }
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
+    if (excl < kk && kk <= excl + sum) {
+        uint32_t run = excl;
+        bool done = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (!done && run + bins[i] >= kk) {
+                atomicMin(&st->tb_run, (uint32_t)(tid * 16 + i));
+                done = true;
+            }
+            run += bins[i];
+        }
+    }
 }
 
 template <int HD>
@@ -149,65 +215,170 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
         wcnt += (uint32_t)__popcll(mask);
         tb = tb_next;
     }
-    if (lane == 0) s_wcnt[wave] = wcnt;
-    __syncthreads();
-
-    // append this block's survivors to the unit's list: one returning atomic per
-    // block, in flight while the histogram is flushed
-    uint32_t wbase = 0, cnt = 0;
-#pragma unroll
-    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
-        if (w2 < wave) wbase += s_wcnt[w2];
-        cnt += s_wcnt[w2];
-    }
-    if (tid == 0) s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
-    uint32_t *hu = hist + (int64_t)unit * DC_HIST_BINS;
-    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
-        const uint32_t c = lhist[i];
-        if (c) atomicAdd(&hu[i], c);
-    }
-    __syncthreads();
-    {
-        uint2 *dst = surv + (int64_t)unit * n_rows + s_base + wbase;
-        for (uint32_t i = lane; i < wcnt; i += 64) dst[i] = wstage[i];
-    }
-    // A few blocks per unit refresh the running threshold from whatever part of
-    // the histogram is visible: every 4th small block, every 8th large one.
-    // Staleness only loosens the bound.
+    // every 4th small block and every 8th large one refresh the running threshold
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
-    if (!refresh) return;
+    prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
+                       surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
+}
 
-    // Coalesced, L2-bypassing read of the unit's histogram into LDS (lhist is
-    // free again), then 16 adjacent bins per thread.
+// sum over aligned groups of LPR lanes (4, 8 or 16)
+template <int LPR>
+__device__ __forceinline__ float sketch_group_sum(float v) {
+    if (LPR == 4) {
+        v += __builtin_amdgcn_update_dpp(0.0f, v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+        v += __builtin_amdgcn_update_dpp(0.0f, v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+        return v;
+    }
+    return dc_group_sum<(LPR == 8 ? 8 : 16)>(v);
+}
+
+// 16 code bytes (value + 128) times 16 weights, added to acc
+__device__ __forceinline__ float sketch_dot16(const uint4 &c, const float (&w)[16], float acc) {
+    const uint32_t x[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc = fmaf((float)(x[i] & 0xffu), w[4 * i + 0], acc);
+        acc = fmaf((float)((x[i] >> 8) & 0xffu), w[4 * i + 1], acc);
+        acc = fmaf((float)((x[i] >> 16) & 0xffu), w[4 * i + 2], acc);
+        acc = fmaf((float)(x[i] >> 24), w[4 * i + 3], acc);
+    }
+    return acc;
+}
+
+// Scan of the 8-bit sketch of the keys.  Row i of a unit is stored as codes
+// u_id = c_id + 128 with k_id = a_d * c_id + e_id, |e_id| <= r_d (a: `scale`,
+// r: `resid`, both per unit and channel).  The scan computes
+//   approx_i = sum_d (q_d a_d) c_id,   |s_i - approx_i| <= E' for every row,
+//   E' = sum_d |q_d| r_d + fp32 slack,
+// where s_i is the fp32 score the exact kernels produce.  With A_k the k-th
+// largest approx, every member of the exact top-k has approx_i >= A_k - 2E' - Q
+// (Q: one quantisation step of the reference key in DC_MODE_REF_DIST, where equal
+// keys of unequal scores tie).  So rows are histogrammed by bucket(approx_i), which
+// yields the bucket of A_k exactly as in score_prune_kernel, and a row is kept when
+// bucket(approx_i + margin) is not worse than the running threshold bucket,
+// margin = 2E' + Q.  The kept rows are rescored exactly by rescore_kernel.
+template <int HD>
+__global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
+    const uint8_t *__restrict__ C, const uint16_t *__restrict__ Q, const float *__restrict__ scale,
+    const float *__restrict__ resid, uint32_t *__restrict__ hist, UnitState *__restrict__ state,
+    uint2 *__restrict__ surv, int n_units, int n_h, int n_rows, int64_t cb, int64_t ch, int64_t cr,
+    int q_group, int mode, int k_eff, int small_chunks, int big_steps) {
+    constexpr int LPR = HD / 16;  // lanes per row, 16 code bytes each
+    __shared__ uint32_t lhist[DC_HIST_BINS];
+    __shared__ uint2 stage[kStage];
+    __shared__ uint32_t wtot[kThreads / 64 + 1];
+    __shared__ uint32_t s_wcnt[kThreads / 64];
+    __shared__ uint32_t s_base;
+
+    const int unit = blockIdx.x % n_units;
+    const int chunk = blockIdx.x / n_units;
+    const int b = unit / n_h, h = unit % n_h;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int grp = lane / LPR, col = lane % LPR;
+
+    const bool small = chunk < small_chunks;
+    const int big_chunks = (int)(gridDim.x / n_units) - small_chunks;
+    const int big_id = small ? 0 : (int)(((int64_t)(chunk - small_chunks) + (int64_t)unit * 7) % big_chunks);
+    const int64_t block_row0 =
+        small ? (int64_t)chunk * kRowsPerBlockStep
+              : (int64_t)small_chunks * kRowsPerBlockStep + (int64_t)big_id * big_steps * kRowsPerBlockStep;
+    const int steps = small ? 1 : big_steps;
+
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
+
+    const uint8_t *Cu = C + b * cb + h * ch + col * 16;
+    UnitState *st = state + unit;
+    const int last = n_rows - 1;
+    uint32_t tb = load_relaxed(&st->tb_run);
+
+    // this lane's 16 weights q_d * a_d, the bias of the +128 code offset, and the margin
+    float w[16];
+    float bias, margin;
     {
-        const unsigned long long *h64 = reinterpret_cast<const unsigned long long *>(hu);
-        unsigned long long *l64 = reinterpret_cast<unsigned long long *>(lhist);
-        for (int i = tid; i < DC_HIST_BINS / 2; i += kThreads)
-            l64[i] = __hip_atomic_load(h64 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    uint32_t bins[16];
-    uint32_t sum = 0;
+        float qv[16];
+        {
+            float t[8];
+            dc_load_query<HD>(Q, unit, q_group, 2 * col, t);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        bins[i] = lhist[tid * 16 + i];
-        sum += bins[i];
-    }
-    uint32_t total;
-    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
-    const uint32_t kk = (uint32_t)k_eff;
-    if (excl < kk && kk <= excl + sum) {
-        uint32_t run = excl;
-        bool done = false;
+            for (int i = 0; i < 8; ++i) qv[i] = t[i];
+            dc_load_query<HD>(Q, unit, q_group, 2 * col + 1, t);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            if (!done && run + bins[i] >= kk) {
-                atomicMin(&st->tb_run, (uint32_t)(tid * 16 + i));
-                done = true;
-            }
-            run += bins[i];
+            for (int i = 0; i < 8; ++i) qv[8 + i] = t[i];
         }
+        const float4 *ap = reinterpret_cast<const float4 *>(scale + (int64_t)unit * HD + col * 16);
+        const float4 *rp = reinterpret_cast<const float4 *>(resid + (int64_t)unit * HD + col * 16);
+        float wsum = 0.f, wabs = 0.f, e = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 a4 = ap[i], r4 = rp[i];
+            const float av[4] = {a4.x, a4.y, a4.z, a4.w}, rv[4] = {r4.x, r4.y, r4.z, r4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float ww = qv[4 * i + j] * av[j];
+                w[4 * i + j] = ww;
+                wsum += ww;
+                wabs += fabsf(ww);
+                e += fabsf(qv[4 * i + j]) * rv[j];
+            }
+        }
+        bias = -128.0f * wsum;
+        wabs = sketch_group_sum<LPR>(wabs);
+        e = sketch_group_sum<LPR>(e);
+        margin = dc_sketch_margin(e, wabs, mode);
     }
+    if (chunk == 0 && tid == 0) st->margin = __float_as_uint(margin);
+    __syncthreads();
+
+    uint2 *wstage = stage + wave * (kBigSteps * 64);
+    uint32_t wcnt = 0;
+    const unsigned long long lt = (1ull << lane) - 1ull;
+
+    // Two steps (2 x 64 rows of this wave) are loaded together: a code row is half as
+    // long as a key row, so it takes twice the rows to keep as many bytes in flight.
+    for (int step = 0; step < steps; step += 2) {
+        const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
+        if (row0 >= n_rows) break;  // wave-uniform; no barrier inside the loop
+        const bool two = step + 1 < steps;
+        uint4 cv[2][LPR];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            if (s2 == 0 || two) {
+#pragma unroll
+                for (int j = 0; j < LPR; ++j) {
+                    int64_t r = row0 + (int64_t)s2 * kRowsPerBlockStep + grp * LPR + j;
+                    r = r > last ? last : r;
+                    cv[s2][j] = *reinterpret_cast<const uint4 *>(Cu + r * cr);
+                }
+            }
+        }
+        uint32_t tb_next = tb;
+        if (step + 2 < steps) tb_next = load_relaxed(&st->tb_run);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            if (s2 == 0 || two) {
+                float mine = 0.f;
+#pragma unroll
+                for (int j = 0; j < LPR; ++j) {
+                    const float p = sketch_group_sum<LPR>(sketch_dot16(cv[s2][j], w, bias));
+                    mine = (col == j) ? p : mine;
+                }
+                const int64_t myrow = row0 + (int64_t)s2 * kRowsPerBlockStep + lane;
+                const bool valid = myrow < n_rows;
+                const uint32_t lb = dc_score_bucket(mine);
+                const bool keep = valid && dc_score_bucket(mine + margin) <= tb;
+                if (keep) atomicAdd(&lhist[lb], 1u);
+                const unsigned long long mask = __ballot(keep);
+                if (keep)
+                    wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+                wcnt += (uint32_t)__popcll(mask);
+            }
+        }
+        tb = tb_next;
+    }
+    const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
+    prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
+                       surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
 }
 
 // Exact threshold bucket of a unit from its complete histogram: the bucket that
@@ -340,12 +511,116 @@ __global__ __launch_bounds__(kThreads) void classify_kernel(
     }
 }
 
+// Second pass of the sketch path.  Several blocks per unit split the list the
+// sketch scan left ((id, approx) pairs): a row stays a candidate when
+// bucket(approx + margin) is not worse than the exact bucket of the k-th largest
+// approx; candidates get their exact fp32 score from the bf16 row, computed lane for
+// lane as score_kernel computes it, and go to a second histogram and list, from
+// which classify_kernel and select_finish_kernel pick the top-k as usual.
+constexpr int kRescoreBatch = 4;
+
+template <int HD>
+__global__ __launch_bounds__(kThreads) void rescore_kernel(
+    const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, const uint32_t *__restrict__ hist1,
+    const UnitState *__restrict__ state1, const uint2 *__restrict__ surv1, uint32_t *__restrict__ hist2,
+    UnitState *__restrict__ state2, uint2 *__restrict__ surv2, int n_units, int n_h, int n_rows,
+    int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int nblk) {
+    constexpr int LPR = HD / 8;
+    constexpr int GROUPS = kThreads / LPR;
+    constexpr uint32_t kPer = kRescoreBatch * kThreads;
+    __shared__ uint32_t lhist[DC_HIST_BINS];
+    __shared__ uint32_t cid[kPer];
+    __shared__ float csc[kPer];
+    __shared__ uint32_t wtot[kThreads / 64 + 1];
+    __shared__ uint32_t sres[2];
+    __shared__ uint32_t s_base;
+    const int unit = blockIdx.x % n_units;
+    const int blk = blockIdx.x / n_units;
+    const int b = unit / n_h, h = unit % n_h;
+    const int tid = threadIdx.x;
+    const int grp = tid / LPR, col = tid % LPR;
+    const UnitState *st1 = state1 + unit;
+    uint32_t n_s = st1->surv_cnt;
+    if (n_s > (uint32_t)n_rows) n_s = n_rows;
+    const uint32_t per = ((n_s + (uint32_t)nblk - 1) / (uint32_t)nblk + kPer - 1) / kPer * kPer;
+    const uint32_t lo = (uint32_t)blk * per;
+    uint32_t hi = lo + per;
+    if (hi > n_s) hi = n_s;
+    if (lo >= n_s) return;
+
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
+    uint32_t tb, c_less;
+    unit_threshold(hist1 + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
+    const float margin = __uint_as_float(st1->margin);
+    float q[8];
+    dc_load_query<HD>(Q, unit, q_group, col, q);
+    const uint16_t *Ku = K + b * sb + h * sh + col * 8;
+    const uint2 *su = surv1 + (int64_t)unit * n_rows;
+    uint2 *du = surv2 + (int64_t)unit * n_rows;
+    UnitState *st2 = state2 + unit;
+
+    for (uint32_t i0 = lo; i0 < hi; i0 += kPer) {
+        uint2 p[kRescoreBatch];
+        uint32_t pass = 0;
+#pragma unroll
+        for (int j = 0; j < kRescoreBatch; ++j) {
+            const uint32_t i = i0 + j * kThreads + tid;
+            p[j] = make_uint2(0u, 0u);
+            if (i < hi) {
+                p[j] = su[i];
+                if (dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
+            }
+        }
+        uint32_t n_c;
+        uint32_t pos = block_excl_scan<kThreads>(__popc(pass), wtot, &n_c);
+#pragma unroll
+        for (int j = 0; j < kRescoreBatch; ++j)
+            if (pass & (1u << j)) cid[pos++] = p[j].x;
+        // the list slot is reserved now and looked at after the rows are scored
+        uint32_t base_reg = 0;
+        if (tid == 0 && n_c) base_reg = atomicAdd(&st2->surv_cnt, n_c);
+        __syncthreads();
+        // exact scores: one LPR-lane group per row, four rows of a group in flight
+        for (uint32_t j0 = 0; j0 < n_c; j0 += GROUPS * 4) {
+            uint4 wv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                uint32_t j = j0 + u * GROUPS + grp;
+                j = j < n_c ? j : n_c - 1;
+                wv[u] = *reinterpret_cast<const uint4 *>(Ku + (int64_t)cid[j] * sr);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t j = j0 + u * GROUPS + grp;
+                const float sc = dc_group_sum<LPR>(dc_dot8(wv[u], q, 0.f));
+                if (col == 0 && j < n_c) {
+                    csc[j] = sc;
+                    uint32_t key, bucket;
+                    dc_key_bucket(sc, mode, key, bucket);
+                    atomicAdd(&lhist[bucket], 1u);
+                }
+            }
+        }
+        if (tid == 0) s_base = base_reg;
+        __syncthreads();
+        for (uint32_t i = tid; i < n_c; i += kThreads)
+            du[s_base + i] = make_uint2(cid[i], __float_as_uint(csc[i]));
+        __syncthreads();  // cid, csc and s_base are rewritten by the next batch
+    }
+    uint32_t *hu = hist2 + (int64_t)unit * DC_HIST_BINS;
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
+        const uint32_t c = lhist[i];
+        if (c) atomicAdd(&hu[i], c);
+    }
+}
+
 // One block per unit: radix select among the candidates of the threshold bucket
 // fills idx_out[c_less, k).  Leaves the unit's list cursors at zero.
 __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     uint32_t *__restrict__ hist, UnitState *__restrict__ state, uint32_t *__restrict__ cand_key,
     uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out, int64_t idx_stride,
-    uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int reinit) {
+    uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int reinit, uint32_t *__restrict__ hist_b,
+    UnitState *__restrict__ state_b) {
     __shared__ uint32_t lh[kRadixBins];
     __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
     __shared__ uint32_t sres[4];
@@ -386,11 +661,19 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
         // leave the unit's histogram and threshold ready for the next scan
         uint4 *hz = reinterpret_cast<uint4 *>(hist + (int64_t)unit * DC_HIST_BINS);
         hz[tid] = make_uint4(0u, 0u, 0u, 0u);
+        if (hist_b) {  // the sketch scan's own histogram and counters
+            hz = reinterpret_cast<uint4 *>(hist_b + (int64_t)unit * DC_HIST_BINS);
+            hz[tid] = make_uint4(0u, 0u, 0u, 0u);
+        }
     }
     if (tid == 0) {
         if (reinit) {
             st->tb_run = DC_HIST_BINS;
             st->surv_cnt = 0;
+            if (state_b) {
+                state_b[unit].tb_run = DC_HIST_BINS;
+                state_b[unit].surv_cnt = 0;
+            }
         }
         st->win_cnt = 0;
         st->cand_cnt = 0;
@@ -467,10 +750,39 @@ FusedWs carve_fused(void *base, int n_units, int n_rows, int k) {
     return w;
 }
 
+// the sketch path adds a second histogram, state array and list (the exact pass)
+struct SketchWs {
+    FusedWs f;
+    uint32_t *hist2;
+    UnitState *state2;
+    uint2 *surv2;
+    size_t bytes;
+};
+
+SketchWs carve_sketch(void *base, int n_units, int n_rows, int k) {
+    SketchWs w;
+    w.f = carve_fused(base, n_units, n_rows, k);
+    char *p = (char *)base;
+    size_t off = w.f.bytes;
+    const size_t nu = n_units > 0 ? n_units : 0, nr = n_rows > 0 ? n_rows : 0;
+    w.hist2 = (uint32_t *)(p + off);
+    off += dc_align_up(nu * DC_HIST_BINS * 4, 256);
+    w.state2 = (UnitState *)(p + off);
+    off += dc_align_up(nu * sizeof(UnitState), 256);
+    w.surv2 = (uint2 *)(p + off);
+    off += dc_align_up(nu * nr * 8, 256);
+    w.bytes = off;
+    return w;
+}
+
 }  // namespace
 
 extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k) {
     return carve_fused(nullptr, n_units, n_rows, k).bytes;
+}
+
+extern "C" size_t dc_sketch_select_workspace_bytes(int n_units, int n_rows, int k) {
+    return carve_sketch(nullptr, n_units, n_rows, k).bytes;
 }
 
 namespace {
@@ -557,6 +869,36 @@ extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_
     return DC_OK;
 }
 
+namespace {
+
+// classify + finish (+ sort) on one (histogram, state, list) triple; hist_b/state_b:
+// a second histogram and state array that the finish kernel re-zeroes as well
+int launch_select(const char *who, uint32_t *hist, UnitState *state, const uint2 *surv, const FusedWs &w,
+                  uint32_t *idx_out, int64_t idx_unit_stride, int n_units, int n_rows, int k_eff, int mode,
+                  int order, int reinit, uint32_t *hist_b, UnitState *state_b, hipStream_t st) {
+    uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
+    // blocks per unit for the classify pass: one per 4096 rows of context, as long as
+    // the grid stays near 2048 blocks
+    int nblk = (n_rows + 4095) / 4096;
+    const int cap = n_units >= 2048 ? 1 : 2048 / n_units;
+    if (nblk > cap) nblk = cap;
+    if (nblk < 1) nblk = 1;
+    hipLaunchKernelGGL(classify_kernel, dim3((unsigned)n_units * (unsigned)nblk), dim3(kThreads), 0, st,
+                       hist, state, surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys,
+                       n_units, n_rows, k_eff, mode, nblk);
+    DC_CHECK_LAUNCH(who);
+    hipLaunchKernelGGL(select_finish_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, hist, state,
+                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows, k_eff, reinit,
+                       hist_b, state_b);
+    DC_CHECK_LAUNCH(who);
+    if (order != DC_ORDER_ANY)
+        return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
+                                k_eff, mode, order, st);
+    return DC_OK;
+}
+
+}  // namespace
+
 extern "C" int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int n_units, int n_rows,
                                 int budget, int mode, int order, int reinit, void *workspace,
                                 size_t workspace_bytes, void *stream) {
@@ -570,25 +912,8 @@ extern "C" int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int 
     FusedWs w;
     int rc = check_ws("dc_sparse_select", workspace, workspace_bytes, n_units, n_rows, budget, &w);
     if (rc) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
-    // blocks per unit for the classify pass: one per 4096 rows of context, as long as
-    // the grid stays near 2048 blocks
-    int nblk = (n_rows + 4095) / 4096;
-    const int cap = n_units >= 2048 ? 1 : 2048 / n_units;
-    if (nblk > cap) nblk = cap;
-    if (nblk < 1) nblk = 1;
-    hipLaunchKernelGGL(classify_kernel, dim3((unsigned)n_units * (unsigned)nblk), dim3(kThreads), 0, st,
-                       w.hist, w.state, w.surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride,
-                       sel_keys, n_units, n_rows, k_eff, mode, nblk);
-    DC_CHECK_LAUNCH("dc_sparse_select");
-    hipLaunchKernelGGL(select_finish_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.hist, w.state,
-                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows, k_eff, reinit);
-    DC_CHECK_LAUNCH("dc_sparse_select");
-    if (order != DC_ORDER_ANY)
-        return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
-                                k_eff, mode, order, st);
-    return DC_OK;
+    return launch_select("dc_sparse_select", w.hist, w.state, w.surv, w, idx_out, idx_unit_stride, n_units,
+                         n_rows, k_eff, mode, order, reinit, nullptr, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out,
@@ -605,4 +930,90 @@ extern "C" int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_
     if (rc) return rc;
     return dc_sparse_select(idx_out, idx_unit_stride, n_units, n_rows, budget, mode, order, 0, workspace,
                             workspace_bytes, stream);
+}
+
+extern "C" int dc_sketch_select_state_init(int n_units, int n_rows, int budget, void *workspace,
+                                           size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(n_units >= 0 && n_rows >= 0 && budget >= 0, "dc_sketch_select_state_init: bad sizes");
+    if (n_units == 0) return DC_OK;
+    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
+               "dc_sketch_select_state_init: workspace must be non-null and 256-byte aligned");
+    const SketchWs w = carve_sketch(workspace, n_units, n_rows, budget);
+    if (workspace_bytes < w.bytes) {
+        dc_set_error("dc_sketch_select_state_init: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
+        return DC_ENOMEM;
+    }
+    const int64_t n = (int64_t)n_units * DC_HIST_BINS;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    hipLaunchKernelGGL(init_state_kernel, grid, dim3(256), 0, (hipStream_t)stream, w.f.hist, w.f.state, n_units);
+    DC_CHECK_LAUNCH("dc_sketch_select_state_init");
+    hipLaunchKernelGGL(init_state_kernel, grid, dim3(256), 0, (hipStream_t)stream, w.hist2, w.state2, n_units);
+    DC_CHECK_LAUNCH("dc_sketch_select_state_init");
+    return DC_OK;
+}
+
+extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, const float *scale,
+                                           const float *resid, const void *q, uint32_t *idx_out,
+                                           int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                                           int64_t sb, int64_t sh, int64_t sr, int64_t cb, int64_t ch,
+                                           int64_t cr, int q_group, int budget, int mode, int order,
+                                           int state_ready, void *workspace, size_t workspace_bytes,
+                                           void *ev_scan_begin, void *ev_scan_end, void *stream) {
+    const char *who = "dc_score_select_sketch_bf16";
+    DC_REQUIRE(k && codes && scale && resid && q && idx_out, "%s: null pointer", who);
+    DC_REQUIRE(q_group >= 1, "%s: bad q_group", who);
+    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d not in {64,128,256}", who, hd);
+    DC_REQUIRE(mode == DC_MODE_IP || mode == DC_MODE_REF_DIST, "%s: bad mode %d", who, mode);
+    DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "%s: bad order %d", who, order);
+    DC_REQUIRE(dc_aligned16(k) && dc_aligned16(codes) && dc_aligned16(scale) && dc_aligned16(resid),
+               "%s: k, codes, scale and resid must be 16-byte aligned", who);
+    DC_REQUIRE(sb % 8 == 0 && sh % 8 == 0 && sr % 8 == 0 && sr >= hd,
+               "%s: key strides must be multiples of 8 elements and row_stride >= hd", who);
+    DC_REQUIRE(cb % 16 == 0 && ch % 16 == 0 && cr % 16 == 0 && cr >= hd,
+               "%s: code strides must be multiples of 16 bytes and row_stride >= hd", who);
+    FusedPlan p;
+    int rc = plan_fused(who, n_b, n_h, n_rows, budget, &p);
+    if (rc) return rc;
+    if (p.n_units == 0 || p.k_eff == 0) return DC_OK;
+    DC_REQUIRE(idx_unit_stride >= p.k_eff, "%s: idx_unit_stride < min(budget, n_rows)", who);
+    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
+               "%s: workspace must be non-null and 256-byte aligned", who);
+    const SketchWs w = carve_sketch(workspace, p.n_units, n_rows, budget);
+    if (workspace_bytes < w.bytes) {
+        dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, w.bytes);
+        return DC_ENOMEM;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (!state_ready) {
+        rc = dc_sketch_select_state_init(p.n_units, n_rows, budget, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+    }
+    if (ev_scan_begin) (void)hipEventRecord((hipEvent_t)ev_scan_begin, st);
+#define DC_LAUNCH_SK(HD)                                                                            \
+    hipLaunchKernelGGL(sketch_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st, codes, \
+                       (const uint16_t *)q, scale, resid, w.f.hist, w.f.state, w.f.surv, p.n_units, n_h, \
+                       n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps)
+    if (hd == 64) DC_LAUNCH_SK(64);
+    else if (hd == 128) DC_LAUNCH_SK(128);
+    else DC_LAUNCH_SK(256);
+#undef DC_LAUNCH_SK
+    DC_CHECK_LAUNCH(who);
+    if (ev_scan_end) (void)hipEventRecord((hipEvent_t)ev_scan_end, st);
+    // blocks per unit of the exact pass: one per 2048 rows of context, grid near 2048 blocks
+    int nblk = (n_rows + 2047) / 2048;
+    const int cap = p.n_units >= 2048 ? 1 : 2048 / p.n_units;
+    if (nblk > cap) nblk = cap;
+    if (nblk < 1) nblk = 1;
+#define DC_LAUNCH_RS(HD)                                                                              \
+    hipLaunchKernelGGL(rescore_kernel<HD>, dim3((unsigned)p.n_units * (unsigned)nblk), dim3(kThreads), 0, \
+                       st, (const uint16_t *)k, (const uint16_t *)q, w.f.hist, w.f.state, w.f.surv,       \
+                       w.hist2, w.state2, w.surv2, p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode,     \
+                       p.k_eff, nblk)
+    if (hd == 64) DC_LAUNCH_RS(64);
+    else if (hd == 128) DC_LAUNCH_RS(128);
+    else DC_LAUNCH_RS(256);
+#undef DC_LAUNCH_RS
+    DC_CHECK_LAUNCH(who);
+    return launch_select(who, w.hist2, w.state2, w.surv2, w.f, idx_out, idx_unit_stride, p.n_units, n_rows,
+                         p.k_eff, mode, order, 1, w.f.hist, w.f.state, st);
 }

@@ -131,6 +131,48 @@ int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out, int64_
                          int mode, int order, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same selection from an 8-bit sketch of the keys: half the HBM bytes of the
+ * bf16 scan, identical ids.  The sketch of a store is one byte per key element
+ * plus, per unit and channel d, a scale a_d and a residual bound r_d with
+ *   k[i, d] = a_d * (codes[i, d] - 128) + e,  |e| <= r_d  for every sketched row.
+ * dc_score_select_sketch_bf16 scans the codes, keeps every row whose approximate
+ * score plus a margin derived from q, a, r and the fp32 rounding of both
+ * evaluations can still reach the k-th best, recomputes the exact fp32 score of
+ * those rows from the bf16 keys with the arithmetic of dc_score_bf16, and selects
+ * among them as dc_sparse_select does: the result is the exact top-k of the bf16
+ * keys (ties -> lower index) whatever the data; only the running time depends on
+ * how well the sketch fits.  No counterpart in the reference, whose exact scan
+ * (diffcache_cpu/src/nsw.rs:592-630) reads every key; same results as that scan.
+ *
+ *   dc_sketch_build_bf16   sketches rows [0, n_rows) of every unit starting at `k`
+ *     (pass pointers to the first row to sketch; codes has its own byte strides,
+ *     multiples of 16, base 16-byte aligned; scale and resid are (n_b*n_h, hd) fp32).
+ *     keep_scale == 0: scales are fitted to these rows (per-channel max / 127) and
+ *     the residual bounds start from zero -- call it on the whole region at prefill.
+ *     keep_scale != 0: the existing scales are used (values outside their range are
+ *     clamped) and the residual bounds are raised where needed -- call it on rows
+ *     appended later (replaces nothing in the reference; goes with lib.rs:352-369).
+ *   dc_score_select_sketch_bf16   arguments as dc_score_select_bf16 plus the sketch;
+ *     state_ready as in dc_layer_args.select_state_ready; the optional event pair is
+ *     recorded around the scan of the codes.
+ */
+int dc_sketch_build_bf16(const void *k, uint8_t *codes, float *scale, float *resid, int n_b, int n_h,
+                         int n_rows, int hd, int64_t k_batch_stride, int64_t k_head_stride,
+                         int64_t k_row_stride, int64_t c_batch_stride, int64_t c_head_stride,
+                         int64_t c_row_stride, int keep_scale, void *stream);
+size_t dc_sketch_select_workspace_bytes(int n_units, int n_rows, int budget);
+int dc_sketch_select_state_init(int n_units, int n_rows, int budget, void *workspace,
+                                size_t workspace_bytes, void *stream);
+int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, const float *scale,
+                                const float *resid, const void *q, uint32_t *idx_out,
+                                int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                                int64_t k_batch_stride, int64_t k_head_stride, int64_t k_row_stride,
+                                int64_t c_batch_stride, int64_t c_head_stride, int64_t c_row_stride,
+                                int q_group, int budget, int mode, int order, int state_ready,
+                                void *workspace, size_t workspace_bytes, void *ev_scan_begin,
+                                void *ev_scan_end, void *stream);
+
+/*
  * Copy selected K and V rows into dense output buffers.
  * For unit (b, h) and j < n_idx:
  *   out_k[b, h, j, :] = k[b, h, row_offset + idx[u, j], :]   (same for v)
@@ -226,6 +268,12 @@ typedef struct dc_layer_args {
                              the init kernel is skipped */
     void *ev_scan_begin;  /* optional hipEvent_t pair recorded on `stream` right before and */
     void *ev_scan_end;    /* right after the scan kernel (for timing it in place), or NULL */
+    const uint8_t *sketch_codes; /* NULL, or the sketch of the K store (row 0 = store row 0): the
+                             streaming select then scans the codes (dc_score_select_sketch_bf16);
+                             needs scores == NULL */
+    const float *sketch_scale;   /* (n_b*n_h, hd) */
+    const float *sketch_resid;   /* (n_b*n_h, hd) */
+    int64_t sketch_batch_stride, sketch_head_stride, sketch_row_stride; /* bytes */
 } dc_layer_args;
 
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,

@@ -268,12 +268,141 @@ def test_streaming_select_full_size_unit(mode):
     check_streaming(k, q, 4, n - 68, 2048, mode, hip.ORDER_BEST)
 
 
+def test_streaming_select_tie_groups_across_the_threshold():
+    # identical rows give exactly equal scores: a 3000-way tie for the last slots of a 2048
+    # budget (more than one block's worth of candidates), and a 600-way tie in a second unit
+    rng = np.random.default_rng(31)
+    b, h, hd, n = 1, 2, 128, 50000
+    k = rand_bf16(rng, b, h, n, hd)
+    q = rand_bf16(rng, b, h, hd)
+    qf = orc.bf16_to_f32(q)
+    strong = orc.f32_to_bf16(np.sign(qf) * 0.75)          # a row every query scores highly
+    pos0 = rng.choice(n, 3000, replace=False)
+    pos1 = rng.choice(n, 600, replace=False)
+    k[0, 0, pos0] = strong[0, 0]
+    k[0, 1, pos1] = strong[0, 1]
+    for mode in (0, 1):
+        check_streaming(k, q, 0, n, 2048, mode, hip.ORDER_BEST)
+        check_streaming(k, q, 0, n, 300, mode, hip.ORDER_INDEX)
+
+
 def test_streaming_select_large_budget():
     rng = np.random.default_rng(5)
     k = rand_bf16(rng, 1, 2, 40000, 128)
     q = rand_bf16(rng, 1, 2, 128)
     check_streaming(k, q, 0, 40000, 9000, hip.MODE_REF_DIST, hip.ORDER_BEST)
     check_streaming(k, q, 0, 40000, 50000, hip.MODE_IP, hip.ORDER_ANY)
+
+
+# ------------------------------------------------------------------ sketch scan + exact rescoring
+
+def check_sketch(k_u16, q_u16, lo, n_rows, budget, mode, order, q_group=1, sketch=None, store=None):
+    """ids of the sketch path == oracle top-k of the dense scores of the same arithmetic"""
+    store = to_dev_bf16(k_u16) if store is None else store
+    qd = to_dev_bf16(q_u16)
+    if sketch is None:
+        sketch = hip.Sketch(store).build(store, lo, n_rows)
+    dense = hip.score(store, qd, lo, n_rows, mode, q_group=q_group).cpu().numpy()
+    ids = hip.score_select_sketch(store, sketch, qd, lo, n_rows, budget, mode, order, q_group=q_group)
+    ids = ids.cpu().numpy().astype(np.uint32)
+    k_eff = min(budget, n_rows)
+    for u in range(dense.shape[0]):
+        want = orc.topk_select(dense[u], budget, mode)
+        got = ids[u, :k_eff]
+        if order == hip.ORDER_BEST:
+            assert np.array_equal(got, want), f"unit {u}"
+        elif order == hip.ORDER_INDEX:
+            assert np.array_equal(got, np.sort(want)), f"unit {u}"
+        else:
+            assert np.array_equal(np.sort(got), np.sort(want)), f"unit {u}"
+    return sketch
+
+
+def test_sketch_codes_and_bounds():
+    # k = a * (code - 128) + e with |e| <= resid for every row and channel; scale = absmax / 127
+    rng = np.random.default_rng(9)
+    b, h, n, hd = 2, 2, 3000, 128
+    scale = np.exp(rng.standard_normal((1, h, 1, hd))).astype(np.float32)
+    k = orc.f32_to_bf16(rng.standard_normal((b, h, n, hd)).astype(np.float32) * scale)
+    k[0, 1, :, 5] = 0                                   # an all-zero channel
+    store = to_dev_bf16(k)
+    sk = hip.Sketch(store).build(store, 7, n - 7)
+    kf = orc.bf16_to_f32(k)[:, :, 7:].reshape(b * h, n - 7, hd)
+    codes = sk.codes.cpu().numpy()[:, :, 7:].reshape(b * h, n - 7, hd).astype(np.float32) - 128
+    a, r = sk.scale.cpu().numpy(), sk.resid.cpu().numpy()
+    amax = np.abs(kf).max(axis=1)
+    assert np.array_equal(a, (amax / np.float32(127)).astype(np.float32))
+    assert np.abs(codes).max() <= 127
+    err = np.abs(kf.astype(np.float64) - a[:, None, :].astype(np.float64) * codes)
+    assert np.all(err <= r[:, None, :] * (1 + 1e-6) + 1e-30)
+    assert np.all(r <= a * 0.5 * (1 + 1e-3) + 1e-30)    # round to nearest inside the fitted range
+    assert a[1, 5] == 0 and r[1, 5] == 0
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("hd", [64, 128, 256])
+@pytest.mark.parametrize("n_rows,budget", [(1, 1), (255, 16), (257, 300), (8193, 1024), (30000, 2048)])
+def test_sketch_select_matches_dense_path(mode, hd, n_rows, budget):
+    rng = np.random.default_rng(hd + n_rows + budget + mode)
+    b, h, lo = 2, 2, 3
+    print(f"sketch mode={mode} hd={hd} n_rows={n_rows} budget={budget}", flush=True)
+    scale = np.exp(rng.standard_normal((1, h, 1, hd))).astype(np.float32)
+    k = orc.f32_to_bf16(rng.standard_normal((b, h, lo + n_rows + 2, hd)).astype(np.float32) * scale)
+    q = rand_bf16(rng, b, h, hd)
+    check_sketch(k, q, lo, n_rows, budget, mode, hip.ORDER_BEST)
+    check_sketch(k, q, lo, n_rows, budget, mode, hip.ORDER_ANY)
+
+
+def test_sketch_select_ties_zero_query_and_group_mean():
+    rng = np.random.default_rng(78)
+    b, h, g, hd, n = 1, 3, 4, 128, 20000
+    k = orc.f32_to_bf16(rng.integers(-2, 3, (b, h, n, hd)).astype(np.float32))
+    q = orc.f32_to_bf16(rng.integers(-1, 2, (b, h * g, hd)).astype(np.float32))
+    q[0, 2 * g:3 * g] = 0                               # everything ties: lowest ids win
+    for mode in (0, 1):
+        check_sketch(k, q, 0, n, 1500, mode, hip.ORDER_BEST, q_group=g)
+        check_sketch(k, q, 0, n, 1500, mode, hip.ORDER_INDEX, q_group=g)
+
+
+def test_sketch_select_rows_outside_the_fitted_range():
+    # rows appended after the scales were fitted, far outside their range, some of them the
+    # best matches: the residual bound grows and the result stays exact
+    rng = np.random.default_rng(79)
+    b, h, hd, n0, n1 = 1, 2, 128, 12000, 16000
+    k = rand_bf16(rng, b, h, n1, hd)
+    q = rand_bf16(rng, b, h, hd)
+    kf = orc.bf16_to_f32(k)
+    qf = orc.bf16_to_f32(q)
+    kf[0, :, n0:n0 + 50] *= 40.0                                  # large rows, random direction
+    kf[0, :, n0 + 50:n0 + 60] = 30.0 * np.sign(qf[0, :, None, :])  # large rows aligned with q
+    k = orc.f32_to_bf16(kf)
+    store = to_dev_bf16(k)
+    sk = hip.Sketch(store).build(store, 0, n0)
+    sk.build(store, n0, n1 - n0, keep_scale=True)
+    assert float(sk.resid.max()) > 10.0
+    for mode in (0, 1):
+        check_sketch(k, q, 0, n1, 512, mode, hip.ORDER_BEST, sketch=sk, store=store)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_sketch_select_full_size_unit(mode):
+    # benchmark shape: 131004-row region, k 2048, keys with outlier channels; 8 units, twice on
+    # one workspace (the second call relies on the state the first one leaves behind)
+    rng = np.random.default_rng(223 + mode)
+    b, h, hd, n = 1, 8, 128, 131072
+    scale = np.exp(rng.standard_normal((1, h, 1, hd))).astype(np.float32)
+    k = orc.f32_to_bf16(rng.standard_normal((b, h, n, hd)).astype(np.float32) * scale)
+    q = rand_bf16(rng, b, h, hd)
+    store, qd = to_dev_bf16(k), to_dev_bf16(q)
+    sk = hip.Sketch(store).build(store, 4, n - 68)
+    check_sketch(k, q, 4, n - 68, 2048, mode, hip.ORDER_BEST, sketch=sk, store=store)
+    ws = hip.alloc_workspace(hip.sketch_select_workspace_bytes(b * h, n - 68, 2048), DEV)
+    a = hip.score_select_sketch(store, sk, qd, 4, n - 68, 2048, mode, hip.ORDER_INDEX, workspace=ws).clone()
+    q2 = to_dev_bf16(rand_bf16(rng, b, h, hd))
+    hip.score_select_sketch(store, sk, q2, 4, n - 68, 2048, mode, hip.ORDER_INDEX, workspace=ws, state_ready=True)
+    c = hip.score_select_sketch(store, sk, qd, 4, n - 68, 2048, mode, hip.ORDER_INDEX, workspace=ws,
+                                state_ready=True)
+    assert torch.equal(a, c)
 
 
 # ------------------------------------------------------------------ gather rows / kv maintenance
