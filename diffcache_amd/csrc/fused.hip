@@ -32,7 +32,7 @@ constexpr int kRowsPerBlockStep = 256;
 constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
-constexpr int kCandLds = 4096;
+constexpr int kCandLds = 8192;
 
 // tb_run is polled by every wave of the scan while surv_cnt takes returning
 // atomics; they sit in separate 128-byte lines because polling a line that is
@@ -515,22 +515,22 @@ __global__ __launch_bounds__(kThreads) void classify_kernel(
 // sketch scan left ((id, approx) pairs): a row stays a candidate when
 // bucket(approx + margin) is not worse than the exact bucket of the k-th largest
 // approx; candidates get their exact fp32 score from the bf16 row, computed lane for
-// lane as score_kernel computes it, and go to a second histogram and list, from
-// which classify_kernel and select_finish_kernel pick the top-k as usual.
+// lane as score_kernel computes it, and their (key, id) go to the unit's candidate
+// list, from which select_finish_kernel picks the k best (c_less = 0: the list
+// holds every member of the top-k).
 constexpr int kRescoreBatch = 4;
 
 template <int HD>
 __global__ __launch_bounds__(kThreads) void rescore_kernel(
-    const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, const uint32_t *__restrict__ hist1,
-    const UnitState *__restrict__ state1, const uint2 *__restrict__ surv1, uint32_t *__restrict__ hist2,
-    UnitState *__restrict__ state2, uint2 *__restrict__ surv2, int n_units, int n_h, int n_rows,
-    int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int nblk) {
+    const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, const uint32_t *__restrict__ hist,
+    UnitState *__restrict__ state, const uint2 *__restrict__ surv, uint32_t *__restrict__ cand_key,
+    uint32_t *__restrict__ cand_idx, int n_units, int n_h, int n_rows, int64_t sb, int64_t sh,
+    int64_t sr, int q_group, int mode, int k_eff, int nblk) {
     constexpr int LPR = HD / 8;
     constexpr int GROUPS = kThreads / LPR;
     constexpr uint32_t kPer = kRescoreBatch * kThreads;
-    __shared__ uint32_t lhist[DC_HIST_BINS];
     __shared__ uint32_t cid[kPer];
-    __shared__ float csc[kPer];
+    __shared__ uint32_t ckey[kPer];
     __shared__ uint32_t wtot[kThreads / 64 + 1];
     __shared__ uint32_t sres[2];
     __shared__ uint32_t s_base;
@@ -539,8 +539,8 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     const int b = unit / n_h, h = unit % n_h;
     const int tid = threadIdx.x;
     const int grp = tid / LPR, col = tid % LPR;
-    const UnitState *st1 = state1 + unit;
-    uint32_t n_s = st1->surv_cnt;
+    UnitState *st = state + unit;
+    uint32_t n_s = st->surv_cnt;
     if (n_s > (uint32_t)n_rows) n_s = n_rows;
     const uint32_t per = ((n_s + (uint32_t)nblk - 1) / (uint32_t)nblk + kPer - 1) / kPer * kPer;
     const uint32_t lo = (uint32_t)blk * per;
@@ -548,28 +548,35 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     if (hi > n_s) hi = n_s;
     if (lo >= n_s) return;
 
-    for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
+    // the block's first batch of the list is requested before the threshold is worked out
+    const uint2 *su = surv + (int64_t)unit * n_rows;
+    uint2 p[kRescoreBatch];
+#pragma unroll
+    for (int j = 0; j < kRescoreBatch; ++j) {
+        const uint32_t i = lo + j * kThreads + tid;
+        p[j] = make_uint2(0u, 0u);
+        if (i < hi) p[j] = su[i];
+    }
     uint32_t tb, c_less;
-    unit_threshold(hist1 + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
-    const float margin = __uint_as_float(st1->margin);
+    unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
+    if (blk == 0 && tid == 0) st->c_less = 0;
+    const float margin = __uint_as_float(st->margin);
     float q[8];
     dc_load_query<HD>(Q, unit, q_group, col, q);
     const uint16_t *Ku = K + b * sb + h * sh + col * 8;
-    const uint2 *su = surv1 + (int64_t)unit * n_rows;
-    uint2 *du = surv2 + (int64_t)unit * n_rows;
-    UnitState *st2 = state2 + unit;
+    uint32_t *ck = cand_key + (int64_t)unit * n_rows;
+    uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
 
     for (uint32_t i0 = lo; i0 < hi; i0 += kPer) {
-        uint2 p[kRescoreBatch];
         uint32_t pass = 0;
 #pragma unroll
         for (int j = 0; j < kRescoreBatch; ++j) {
             const uint32_t i = i0 + j * kThreads + tid;
-            p[j] = make_uint2(0u, 0u);
-            if (i < hi) {
-                p[j] = su[i];
-                if (dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
+            if (i0 != lo) {
+                p[j] = make_uint2(0u, 0u);
+                if (i < hi) p[j] = su[i];
             }
+            if (i < hi && dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
         }
         uint32_t n_c;
         uint32_t pos = block_excl_scan<kThreads>(__popc(pass), wtot, &n_c);
@@ -578,39 +585,39 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
             if (pass & (1u << j)) cid[pos++] = p[j].x;
         // the list slot is reserved now and looked at after the rows are scored
         uint32_t base_reg = 0;
-        if (tid == 0 && n_c) base_reg = atomicAdd(&st2->surv_cnt, n_c);
+        if (tid == 0 && n_c) base_reg = atomicAdd(&st->cand_cnt, n_c);
         __syncthreads();
-        // exact scores: one LPR-lane group per row, four rows of a group in flight
-        for (uint32_t j0 = 0; j0 < n_c; j0 += GROUPS * 4) {
-            uint4 wv[4];
+        // exact scores: one LPR-lane group per row, kRowsInFlight rows of a group in flight
+        constexpr int kRowsInFlight = 8;
+        for (uint32_t j0 = 0; j0 < n_c; j0 += GROUPS * kRowsInFlight) {
+            uint4 wv[kRowsInFlight];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kRowsInFlight; ++u) {
                 uint32_t j = j0 + u * GROUPS + grp;
                 j = j < n_c ? j : n_c - 1;
                 wv[u] = *reinterpret_cast<const uint4 *>(Ku + (int64_t)cid[j] * sr);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kRowsInFlight; ++u) {
                 const uint32_t j = j0 + u * GROUPS + grp;
                 const float sc = dc_group_sum<LPR>(dc_dot8(wv[u], q, 0.f));
                 if (col == 0 && j < n_c) {
-                    csc[j] = sc;
                     uint32_t key, bucket;
                     dc_key_bucket(sc, mode, key, bucket);
-                    atomicAdd(&lhist[bucket], 1u);
+                    ckey[j] = key;
                 }
             }
         }
         if (tid == 0) s_base = base_reg;
         __syncthreads();
-        for (uint32_t i = tid; i < n_c; i += kThreads)
-            du[s_base + i] = make_uint2(cid[i], __float_as_uint(csc[i]));
-        __syncthreads();  // cid, csc and s_base are rewritten by the next batch
-    }
-    uint32_t *hu = hist2 + (int64_t)unit * DC_HIST_BINS;
-    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
-        const uint32_t c = lhist[i];
-        if (c) atomicAdd(&hu[i], c);
+        for (uint32_t i = tid; i < n_c; i += kThreads) {
+            const uint32_t slot = s_base + i;
+            if (slot < (uint32_t)n_rows) {
+                ck[slot] = ckey[i];
+                ci[slot] = cid[i];
+            }
+        }
+        __syncthreads();  // cid, ckey and s_base are rewritten by the next batch
     }
 }
 
@@ -619,8 +626,7 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
 __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     uint32_t *__restrict__ hist, UnitState *__restrict__ state, uint32_t *__restrict__ cand_key,
     uint32_t *__restrict__ cand_idx, uint32_t *__restrict__ idx_out, int64_t idx_stride,
-    uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int reinit, uint32_t *__restrict__ hist_b,
-    UnitState *__restrict__ state_b) {
+    uint32_t *__restrict__ sel_keys, int n_rows, int k_eff, int reinit) {
     __shared__ uint32_t lh[kRadixBins];
     __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
     __shared__ uint32_t sres[4];
@@ -661,19 +667,11 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
         // leave the unit's histogram and threshold ready for the next scan
         uint4 *hz = reinterpret_cast<uint4 *>(hist + (int64_t)unit * DC_HIST_BINS);
         hz[tid] = make_uint4(0u, 0u, 0u, 0u);
-        if (hist_b) {  // the sketch scan's own histogram and counters
-            hz = reinterpret_cast<uint4 *>(hist_b + (int64_t)unit * DC_HIST_BINS);
-            hz[tid] = make_uint4(0u, 0u, 0u, 0u);
-        }
     }
     if (tid == 0) {
         if (reinit) {
             st->tb_run = DC_HIST_BINS;
             st->surv_cnt = 0;
-            if (state_b) {
-                state_b[unit].tb_run = DC_HIST_BINS;
-                state_b[unit].surv_cnt = 0;
-            }
         }
         st->win_cnt = 0;
         st->cand_cnt = 0;
@@ -750,31 +748,6 @@ FusedWs carve_fused(void *base, int n_units, int n_rows, int k) {
     return w;
 }
 
-// the sketch path adds a second histogram, state array and list (the exact pass)
-struct SketchWs {
-    FusedWs f;
-    uint32_t *hist2;
-    UnitState *state2;
-    uint2 *surv2;
-    size_t bytes;
-};
-
-SketchWs carve_sketch(void *base, int n_units, int n_rows, int k) {
-    SketchWs w;
-    w.f = carve_fused(base, n_units, n_rows, k);
-    char *p = (char *)base;
-    size_t off = w.f.bytes;
-    const size_t nu = n_units > 0 ? n_units : 0, nr = n_rows > 0 ? n_rows : 0;
-    w.hist2 = (uint32_t *)(p + off);
-    off += dc_align_up(nu * DC_HIST_BINS * 4, 256);
-    w.state2 = (UnitState *)(p + off);
-    off += dc_align_up(nu * sizeof(UnitState), 256);
-    w.surv2 = (uint2 *)(p + off);
-    off += dc_align_up(nu * nr * 8, 256);
-    w.bytes = off;
-    return w;
-}
-
 }  // namespace
 
 extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k) {
@@ -782,7 +755,7 @@ extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k
 }
 
 extern "C" size_t dc_sketch_select_workspace_bytes(int n_units, int n_rows, int k) {
-    return carve_sketch(nullptr, n_units, n_rows, k).bytes;
+    return carve_fused(nullptr, n_units, n_rows, k).bytes;  // the same lists serve both paths
 }
 
 namespace {
@@ -871,11 +844,22 @@ extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_
 
 namespace {
 
-// classify + finish (+ sort) on one (histogram, state, list) triple; hist_b/state_b:
-// a second histogram and state array that the finish kernel re-zeroes as well
-int launch_select(const char *who, uint32_t *hist, UnitState *state, const uint2 *surv, const FusedWs &w,
-                  uint32_t *idx_out, int64_t idx_unit_stride, int n_units, int n_rows, int k_eff, int mode,
-                  int order, int reinit, uint32_t *hist_b, UnitState *state_b, hipStream_t st) {
+// finish (+ sort): picks min(k, candidates) from the unit's candidate list
+int launch_finish(const char *who, const FusedWs &w, uint32_t *idx_out, int64_t idx_unit_stride, int n_units,
+                  int n_rows, int k_eff, int mode, int order, int reinit, hipStream_t st) {
+    uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
+    hipLaunchKernelGGL(select_finish_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, w.hist, w.state,
+                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows, k_eff, reinit);
+    DC_CHECK_LAUNCH(who);
+    if (order != DC_ORDER_ANY)
+        return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
+                                k_eff, mode, order, st);
+    return DC_OK;
+}
+
+// classify + finish (+ sort) on the survivor list of score_prune_kernel
+int launch_select(const char *who, const FusedWs &w, uint32_t *idx_out, int64_t idx_unit_stride, int n_units,
+                  int n_rows, int k_eff, int mode, int order, int reinit, hipStream_t st) {
     uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
     // blocks per unit for the classify pass: one per 4096 rows of context, as long as
     // the grid stays near 2048 blocks
@@ -884,17 +868,10 @@ int launch_select(const char *who, uint32_t *hist, UnitState *state, const uint2
     if (nblk > cap) nblk = cap;
     if (nblk < 1) nblk = 1;
     hipLaunchKernelGGL(classify_kernel, dim3((unsigned)n_units * (unsigned)nblk), dim3(kThreads), 0, st,
-                       hist, state, surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys,
+                       w.hist, w.state, w.surv, w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys,
                        n_units, n_rows, k_eff, mode, nblk);
     DC_CHECK_LAUNCH(who);
-    hipLaunchKernelGGL(select_finish_kernel, dim3(n_units), dim3(kFinalThreads), 0, st, hist, state,
-                       w.cand_key, w.cand_idx, idx_out, idx_unit_stride, sel_keys, n_rows, k_eff, reinit,
-                       hist_b, state_b);
-    DC_CHECK_LAUNCH(who);
-    if (order != DC_ORDER_ANY)
-        return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
-                                k_eff, mode, order, st);
-    return DC_OK;
+    return launch_finish(who, w, idx_out, idx_unit_stride, n_units, n_rows, k_eff, mode, order, reinit, st);
 }
 
 }  // namespace
@@ -912,8 +889,8 @@ extern "C" int dc_sparse_select(uint32_t *idx_out, int64_t idx_unit_stride, int 
     FusedWs w;
     int rc = check_ws("dc_sparse_select", workspace, workspace_bytes, n_units, n_rows, budget, &w);
     if (rc) return rc;
-    return launch_select("dc_sparse_select", w.hist, w.state, w.surv, w, idx_out, idx_unit_stride, n_units,
-                         n_rows, k_eff, mode, order, reinit, nullptr, nullptr, (hipStream_t)stream);
+    return launch_select("dc_sparse_select", w, idx_out, idx_unit_stride, n_units, n_rows, k_eff, mode, order,
+                         reinit, (hipStream_t)stream);
 }
 
 extern "C" int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out,
@@ -934,22 +911,7 @@ extern "C" int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_
 
 extern "C" int dc_sketch_select_state_init(int n_units, int n_rows, int budget, void *workspace,
                                            size_t workspace_bytes, void *stream) {
-    DC_REQUIRE(n_units >= 0 && n_rows >= 0 && budget >= 0, "dc_sketch_select_state_init: bad sizes");
-    if (n_units == 0) return DC_OK;
-    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
-               "dc_sketch_select_state_init: workspace must be non-null and 256-byte aligned");
-    const SketchWs w = carve_sketch(workspace, n_units, n_rows, budget);
-    if (workspace_bytes < w.bytes) {
-        dc_set_error("dc_sketch_select_state_init: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
-        return DC_ENOMEM;
-    }
-    const int64_t n = (int64_t)n_units * DC_HIST_BINS;
-    const dim3 grid((unsigned)((n + 255) / 256));
-    hipLaunchKernelGGL(init_state_kernel, grid, dim3(256), 0, (hipStream_t)stream, w.f.hist, w.f.state, n_units);
-    DC_CHECK_LAUNCH("dc_sketch_select_state_init");
-    hipLaunchKernelGGL(init_state_kernel, grid, dim3(256), 0, (hipStream_t)stream, w.hist2, w.state2, n_units);
-    DC_CHECK_LAUNCH("dc_sketch_select_state_init");
-    return DC_OK;
+    return dc_select_state_init(n_units, n_rows, budget, workspace, workspace_bytes, stream);
 }
 
 extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, const float *scale,
@@ -978,7 +940,7 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
     DC_REQUIRE(idx_unit_stride >= p.k_eff, "%s: idx_unit_stride < min(budget, n_rows)", who);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "%s: workspace must be non-null and 256-byte aligned", who);
-    const SketchWs w = carve_sketch(workspace, p.n_units, n_rows, budget);
+    const FusedWs w = carve_fused(workspace, p.n_units, n_rows, budget);
     if (workspace_bytes < w.bytes) {
         dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, w.bytes);
         return DC_ENOMEM;
@@ -991,7 +953,7 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
     if (ev_scan_begin) (void)hipEventRecord((hipEvent_t)ev_scan_begin, st);
 #define DC_LAUNCH_SK(HD)                                                                            \
     hipLaunchKernelGGL(sketch_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st, codes, \
-                       (const uint16_t *)q, scale, resid, w.f.hist, w.f.state, w.f.surv, p.n_units, n_h, \
+                       (const uint16_t *)q, scale, resid, w.hist, w.state, w.surv, p.n_units, n_h,       \
                        n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps)
     if (hd == 64) DC_LAUNCH_SK(64);
     else if (hd == 128) DC_LAUNCH_SK(128);
@@ -1006,14 +968,12 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
     if (nblk < 1) nblk = 1;
 #define DC_LAUNCH_RS(HD)                                                                              \
     hipLaunchKernelGGL(rescore_kernel<HD>, dim3((unsigned)p.n_units * (unsigned)nblk), dim3(kThreads), 0, \
-                       st, (const uint16_t *)k, (const uint16_t *)q, w.f.hist, w.f.state, w.f.surv,       \
-                       w.hist2, w.state2, w.surv2, p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode,     \
-                       p.k_eff, nblk)
+                       st, (const uint16_t *)k, (const uint16_t *)q, w.hist, w.state, w.surv, w.cand_key, \
+                       w.cand_idx, p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode, p.k_eff, nblk)
     if (hd == 64) DC_LAUNCH_RS(64);
     else if (hd == 128) DC_LAUNCH_RS(128);
     else DC_LAUNCH_RS(256);
 #undef DC_LAUNCH_RS
     DC_CHECK_LAUNCH(who);
-    return launch_select(who, w.hist2, w.state2, w.surv2, w.f, idx_out, idx_unit_stride, p.n_units, n_rows,
-                         p.k_eff, mode, order, 1, w.f.hist, w.f.state, st);
+    return launch_finish(who, w, idx_out, idx_unit_stride, p.n_units, n_rows, p.k_eff, mode, order, 1, st);
 }
