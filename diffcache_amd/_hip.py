@@ -18,7 +18,7 @@ MODE_REF_DIST = 1
 ORDER_ANY = 0
 ORDER_BEST = 1
 ORDER_INDEX = 2
-HIST_BINS = 4096
+HIST_BINS = 1024
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdiffcache_hip.so")

@@ -8,7 +8,7 @@
 // a kernel that otherwise streams 256 bytes/row at the read ceiling.
 //
 // score_prune_kernel streams the key rows like score_kernel, bins every key in
-// the unit's 4096-bucket histogram, and keeps a row only if its bucket is not
+// the unit's bucket histogram, and keeps a row only if its bucket is not
 // worse than the unit's running threshold bucket tb_run.  tb_run is the bucket
 // of the k-th best key among the rows histogrammed so far; rows can only be
 // added, so tb_run never undershoots the final threshold bucket and no member
@@ -33,6 +33,8 @@ constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 8192;
+constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
+static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kThreads == DC_HIST_BINS, "bin split");
 
 // tb_run is polled by every wave of the scan while surv_cnt takes returning
 // atomics; they sit in separate 128-byte lines because polling a line that is
@@ -101,7 +103,7 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
     if (!refresh) return;
 
     // Coalesced, L2-bypassing read of the unit's histogram into LDS (lhist is
-    // free again), then 16 adjacent bins per thread.
+    // free again), then kBinsPerThread adjacent bins per thread.
     {
         const unsigned long long *h64 = reinterpret_cast<const unsigned long long *>(hu);
         unsigned long long *l64 = reinterpret_cast<unsigned long long *>(lhist);
@@ -109,11 +111,11 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
             l64[i] = __hip_atomic_load(h64 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    uint32_t bins[16];
+    uint32_t bins[kBinsPerThread];
     uint32_t sum = 0;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        bins[i] = lhist[tid * 16 + i];
+    for (int i = 0; i < kBinsPerThread; ++i) {
+        bins[i] = lhist[tid * kBinsPerThread + i];
         sum += bins[i];
     }
     uint32_t total;
@@ -122,9 +124,9 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
         uint32_t run = excl;
         bool done = false;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < kBinsPerThread; ++i) {
             if (!done && run + bins[i] >= kk) {
-                atomicMin(&st->tb_run, (uint32_t)(tid * 16 + i));
+                atomicMin(&st->tb_run, (uint32_t)(tid * kBinsPerThread + i));
                 done = true;
             }
             run += bins[i];
@@ -392,11 +394,11 @@ __device__ __forceinline__ void unit_threshold(const uint32_t *__restrict__ hu, 
         sres[0] = DC_HIST_BINS;
         sres[1] = 0;
     }
-    uint32_t bins[16];
+    uint32_t bins[kBinsPerThread];
     uint32_t sum = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint4 t = reinterpret_cast<const uint4 *>(hu)[tid * 4 + i];
+    for (int i = 0; i < kBinsPerThread / 4; ++i) {
+        const uint4 t = reinterpret_cast<const uint4 *>(hu)[tid * (kBinsPerThread / 4) + i];
         bins[4 * i + 0] = t.x;
         bins[4 * i + 1] = t.y;
         bins[4 * i + 2] = t.z;
@@ -409,9 +411,9 @@ __device__ __forceinline__ void unit_threshold(const uint32_t *__restrict__ hu, 
         uint32_t run = excl;
         bool done = false;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < kBinsPerThread; ++i) {
             if (!done && run + bins[i] >= kk) {
-                sres[0] = tid * 16 + i;
+                sres[0] = tid * kBinsPerThread + i;
                 sres[1] = run;
                 done = true;
             }
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     if (reinit) {
         // leave the unit's histogram and threshold ready for the next scan
         uint4 *hz = reinterpret_cast<uint4 *>(hist + (int64_t)unit * DC_HIST_BINS);
-        hz[tid] = make_uint4(0u, 0u, 0u, 0u);
+        if (tid < DC_HIST_BINS / 4) hz[tid] = make_uint4(0u, 0u, 0u, 0u);
     }
     if (tid == 0) {
         if (reinit) {

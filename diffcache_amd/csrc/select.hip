@@ -5,7 +5,7 @@
 // the lower id), which is also what DualHeap keeps (dualheap.rs:4-87).
 //
 // Three stages, all streaming or tiny:
-//   1. a 4096-bucket histogram of a monotone 12-bit function of the key (filled
+//   1. a DC_HIST_BINS-bucket histogram of a monotone function of the key (filled
 //      by the scoring kernel's epilogue, or by hist_kernel here);
 //   2. filter_kernel: every block finds the bucket tb holding the k-th key,
 //      emits all ids in buckets < tb (certain members) and the (key, id) pairs
@@ -79,12 +79,15 @@ __global__ __launch_bounds__(kFilterThreads) void filter_kernel(
         s_cless = 0;
     }
     // ---- threshold bucket: the bucket holding the k_eff-th smallest key ----
-    uint32_t bins[16];
+    constexpr int kBinsPerThread = DC_HIST_BINS / kFilterThreads;
+    static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kFilterThreads == DC_HIST_BINS, "bin split");
+    uint32_t bins[kBinsPerThread];
     uint32_t sum = 0;
     {
-        const uint4 *hp = reinterpret_cast<const uint4 *>(hist + (int64_t)unit * DC_HIST_BINS) + tid * 4;
+        const uint4 *hp =
+            reinterpret_cast<const uint4 *>(hist + (int64_t)unit * DC_HIST_BINS) + tid * (kBinsPerThread / 4);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kBinsPerThread / 4; ++i) {
             uint4 t = hp[i];
             bins[4 * i + 0] = t.x;
             bins[4 * i + 1] = t.y;
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(kFilterThreads) void filter_kernel(
             bins[4 * i + 3] = t.w;
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) sum += bins[i];
+        for (int i = 0; i < kBinsPerThread; ++i) sum += bins[i];
     }
     uint32_t total;
     uint32_t excl = block_excl_scan<kFilterThreads>(sum, wtot, &total);
@@ -101,9 +104,9 @@ __global__ __launch_bounds__(kFilterThreads) void filter_kernel(
         uint32_t run = excl;
         bool done = false;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < kBinsPerThread; ++i) {
             if (!done && run + bins[i] >= kk) {
-                s_tb = tid * 16 + i;
+                s_tb = tid * kBinsPerThread + i;
                 s_cless = run;
                 done = true;
             }

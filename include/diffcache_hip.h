@@ -47,7 +47,7 @@ extern "C" {
 #define DC_ENOMEM (-12)   /* workspace too small */
 #define DC_ELAUNCH (-5)   /* hipLaunchKernel failed */
 
-#define DC_HIST_BINS 4096 /* coarse histogram bins per unit used by the select */
+#define DC_HIST_BINS 1024 /* histogram bins per unit used by the select */
 
 /* Library version (DC_VERSION).  Replaces nothing; added for binding checks. */
 int dc_version(void);
