@@ -35,7 +35,7 @@ _DEFAULTS = dict(  # lib.rs:556-566
     use_bruteforce=False, attn_mass_threshold=0.9,
     k_check_seq=[100, 200, 300, 400, 800, 1600, 3200, 6400, 12800, 25600],
 )
-_EXTRA = dict(device="cuda", key_mode="ref_dist", storage=None)  # not in the reference
+_EXTRA = dict(device="cuda", key_mode="ref_dist", storage=None, key_sketch=False)  # not in the reference
 
 _metrics: Dict[str, int] = {}
 _metrics_on = False
@@ -120,6 +120,13 @@ class DiffCacheHIP:
         self._ws: Optional[torch.Tensor] = None
         self._ws_key = None
         self._idx: Optional[torch.Tensor] = None
+        # optional 8-bit sketch of the keys: queries scan it instead of the bf16 rows and
+        # rescore the rows that can still matter; the ids are the same
+        self.sketch: Optional[hip.Sketch] = hip.Sketch(self.keys) if opt["key_sketch"] else None
+
+    def _resketch(self) -> None:
+        if self.sketch is not None and self.ctx_len > 0:
+            self.sketch.build(self.keys, 0, self.ctx_len)
 
     # ------------------------------------------------------------------ ingest
     def prefill(self, keys: ArrayLike, vals: ArrayLike, neighbours: Optional[ArrayLike] = None) -> None:
@@ -135,6 +142,7 @@ class DiffCacheHIP:
         self.keys[:, :, :seq].copy_(k)
         self.vals[:, :, :seq].copy_(v)
         self.ctx_len = seq
+        self._resketch()
 
     def prefill_bshd(self, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
         """Ingest straight from the model layout (bsz, seq, kv_heads, hd) with the
@@ -144,6 +152,7 @@ class DiffCacheHIP:
         hip.ingest_kv(self.keys, key_states, 0)
         hip.ingest_kv(self.vals, value_states, 0)
         self.ctx_len = seq
+        self._resketch()
 
     def insert(self, keys: ArrayLike, vals: ArrayLike) -> None:
         """keys, vals (bsz, kv_heads, hd): append one token (lib.rs:352-369)."""
@@ -154,6 +163,11 @@ class DiffCacheHIP:
         assert tuple(v.shape) == want, f"vals shape {tuple(v.shape)} != {want}"        # lib.rs:354
         assert self.ctx_len < self.max_ctx_len, "index is full"
         hip.append_kv(self.keys, self.vals, k, v, self.ctx_len)
+        if self.sketch is not None:
+            if self.ctx_len == 0:
+                self.sketch.build(self.keys, 0, 1)
+            else:   # keep the fitted scales; the residual bounds grow if the row lies outside them
+                self.sketch.build(self.keys, self.ctx_len, 1, keep_scale=True)
         self.ctx_len += 1
 
     # ------------------------------------------------------------------ query
@@ -181,6 +195,9 @@ class DiffCacheHIP:
             ids = hip.topk_select(scores, ef, self.mode, hip.ORDER_BEST)
             return ids, scores
         ws = self._workspace(self.ctx_len, ef)
+        if self.sketch is not None:
+            return hip.score_select_sketch(self.keys, self.sketch, q.contiguous(), 0, self.ctx_len, ef,
+                                           self.mode, hip.ORDER_BEST, idx_out=self._idx, workspace=ws)
         return hip.score_select(self.keys, q.contiguous(), 0, self.ctx_len, ef, self.mode, hip.ORDER_BEST,
                                 idx_out=self._idx, workspace=ws)
 
@@ -276,3 +293,4 @@ class DiffCacheHIP:
                 self.r_sq[h] = snap["options"]["r_sq"]
         # the reference scans valid nodes only (nsw.rs:601-605), whatever ctx_len says
         self.ctx_len = min(int(ctx_len), n_min if n_min is not None else 0)
+        self._resketch()

@@ -57,6 +57,7 @@ class DiffCache:
         r_sq: List[List[float]],
         key_mode: str = "ref_dist",
         device: str = "cuda",
+        key_sketch: bool = True,
     ) -> None:
         self.num_layers = num_layers
         self.batch_size = batch_size
@@ -94,6 +95,14 @@ class DiffCache:
         self._kslab = torch.zeros(store, device=self.device, dtype=torch.bfloat16)
         self.kstore = [self._kslab[l] for l in range(num_layers)]
         self.vstore = [self._vslab[l] for l in range(num_layers)]
+        # 8-bit sketch of the keys (one byte per element, +25 % memory): the scan reads it
+        # instead of the bf16 keys and rescores the rows that can still matter, with the same
+        # result.  Allocated last: it is the buffer every decode step streams.
+        self.key_sketch = key_sketch
+        self.sketch: List[Optional[hip.Sketch]] = [None] * num_layers
+        if key_sketch:
+            self._cslab = torch.zeros(store, device=self.device, dtype=torch.uint8)
+            self.sketch = [hip.Sketch(self.kstore[l], codes=self._cslab[l]) for l in range(num_layers)]
 
         n_units = batch_size * num_kv_heads
         self.group = num_q_heads // num_kv_heads
@@ -104,7 +113,11 @@ class DiffCache:
                     for _ in range(num_layers)]
         self._ws: Optional[torch.Tensor] = None
         self._ws_rows = -1
-        self._ws_ready = False   # True once a decode_attention call has left the select state ready
+        # The select state inside the workspace is laid out differently by dc_decode_layer and
+        # by the stand-alone select calls, so each route keeps its own "left ready" flag and
+        # clears the other's.
+        self._ws_ready = False        # a decode_attention call has left its select state ready
+        self._hook_ws_ready = False   # a decode_query_kvcache call (sketch route) has
         self._attn_out: Optional[torch.Tensor] = None
         self._prefix0 = kvbuf_prefix_len
         self._suffix0 = kvbuf_suffix_len
@@ -126,6 +139,7 @@ class DiffCache:
                                           self.head_dim, attended), self.device)
             self._ws_rows = region
             self._ws_ready = False
+            self._hook_ws_ready = False
         return self._ws
 
     # ------------------------------------------------------------------ prefill
@@ -148,6 +162,8 @@ class DiffCache:
         self.kvbuf_prefix_len = prefix_len
         self.kvbuf_suffix_len = suffix_len
         self.retrieval_region_len = seq_len - prefix_len - suffix_len
+        if self.key_sketch and self.retrieval_region_len > 0:
+            self.sketch[layer_idx].build(self.kstore[layer_idx], prefix_len, self.retrieval_region_len)
 
         # prefix and suffix rows of the assembled buffer (diffcache.py:164-171)
         b0 = self.retrieval_budget
@@ -192,9 +208,16 @@ class DiffCache:
         if retrieval_len > 0:
             lo, hi = self._region()
             ws = self._ensure_workspace()
-            hip.score_select(self.kstore[layer_idx], self.qbuf, lo, hi - lo, retrieval_len, self.mode,
-                             hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
-            self._ws_ready = False   # the one-shot call does not leave the state initialised
+            if self.key_sketch:
+                hip.score_select_sketch(self.kstore[layer_idx], self.sketch[layer_idx], self.qbuf, lo, hi - lo,
+                                        retrieval_len, self.mode, hip.ORDER_BEST, idx_out=self.idx[layer_idx],
+                                        workspace=ws, state_ready=self._hook_ws_ready)
+                self._hook_ws_ready = True
+            else:
+                hip.score_select(self.kstore[layer_idx], self.qbuf, lo, hi - lo, retrieval_len, self.mode,
+                                 hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
+                self._hook_ws_ready = False   # the one-shot call does not leave the state initialised
+            self._ws_ready = False
         assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
@@ -237,8 +260,10 @@ class DiffCache:
         ws = self._ensure_workspace()
         hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
                          self.kvbuf_suffix_len + 1, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
-                         mode=self.mode, order=order, select_state_ready=self._ws_ready)
+                         mode=self.mode, order=order, select_state_ready=self._ws_ready,
+                         sketch=self.sketch[layer_idx])
         self._ws_ready = True
+        self._hook_ws_ready = False
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
         return out
@@ -302,6 +327,8 @@ class DiffCache:
             layer_path = os.path.join(prefill_cache_path, f"d_l_{layer_idx:03d}")
             self.data_layers[layer_idx].load(layer_path, ctx_len)
             self.data_layers[layer_idx].update_r_sq(self.r_sq[layer_idx])
+            if self.key_sketch and hi > lo:
+                self.sketch[layer_idx].build(self.kstore[layer_idx], lo, hi - lo)
 
     def seq_len(self, layer_idx: int) -> int:
         return self.kvbuf_prefix_len + self.kvbuf_suffix_len + self.retrieval_region_len

@@ -33,6 +33,30 @@ def bf16_close(got_f32, want_f64):
 
 # ---------------------------------------------------------------- DiffCacheHIP
 
+def test_data_layer_with_key_sketch_follows_inserts():
+    """key_sketch=True: same rows as the C restatement of the exact scan, also after rows far
+    outside the range the sketch was fitted to have been inserted."""
+    from diffcache_amd import DiffCacheHIP
+    rng = np.random.default_rng(33)
+    b, hkv, hd, n0 = 1, 2, 128, 600
+    dl = DiffCacheHIP(b, 2, hkv, hd, max_ctx_len=1024, key_sketch=True)
+    keys = orc.f32_to_bf16(rng.integers(-3, 4, (b, hkv, n0, hd)).astype(np.float32))
+    vals = rand_bf16(rng, b, hkv, n0, hd)
+    dl.prefill(keys, vals)
+    extra_k = orc.f32_to_bf16(rng.integers(-60, 61, (8, b, hkv, hd)).astype(np.float32))
+    extra_v = rand_bf16(rng, 8, b, hkv, hd)
+    for i in range(8):
+        dl.insert(extra_k[i], extra_v[i])
+    all_k = np.concatenate([keys, np.transpose(extra_k, (1, 2, 0, 3))], axis=2)
+    all_v = np.concatenate([vals, np.transpose(extra_v, (1, 2, 0, 3))], axis=2)
+    q = orc.f32_to_bf16(rng.integers(-2, 3, (b, hkv, hd)).astype(np.float32))
+    out_k = torch.zeros((b, hkv, 64, hd), dtype=torch.bfloat16, device=DEV)
+    out_v = torch.zeros_like(out_k)
+    dl.query(out_k, out_v, q, 64)
+    ck, cv, _ = cpu_ref.query(all_k, all_v, q, 64)
+    assert np.array_equal(np_u16(out_k), ck) and np.array_equal(np_u16(out_v), cv)
+
+
 def test_data_layer_query_equals_cpu_reference_rows():
     """prefill + query with numpy u16 in/out, the calling convention of
     diffcache.py:147,218-220; integer-valued data makes every fp32 accumulation
@@ -133,9 +157,10 @@ def test_data_layer_save_load_roundtrip(tmp_path):
 
 # ---------------------------------------------------------------- DiffCache
 
-def make_cache(num_layers, b, max_len, hkv, hq, hd, budget, p, s, smax, key_mode="ref_dist"):
+def make_cache(num_layers, b, max_len, hkv, hq, hd, budget, p, s, smax, key_mode="ref_dist",
+               key_sketch=True):
     from diffcache_amd import DiffCache
-    return DiffCache(num_layers=num_layers, batch_size=b, max_length=max_len, num_kv_heads=hkv,
+    return DiffCache(key_sketch=key_sketch, num_layers=num_layers, batch_size=b, max_length=max_len, num_kv_heads=hkv,
                      num_q_heads=hq, head_dim=hd, retrieval_budget=budget, nsw_m=16, nsw_ef_cons=200,
                      kvbuf_prefix_len=p, kvbuf_suffix_len=s, kvbuf_suffix_maxlen=smax,
                      attn_mass_threshold=0.9, k_check_seq=[1048576],
@@ -220,6 +245,33 @@ def test_diffcache_decode_attention_matches_oracle_over_steps(key_mode):
             hist_k[l] = np.concatenate([hist_k[l], np.transpose(nk, (0, 2, 1, 3))], axis=2)
             hist_v[l] = np.concatenate([hist_v[l], np.transpose(nv, (0, 2, 1, 3))], axis=2)
         assert cache.kvbuf_suffix_len == s_len + step + 1
+
+
+def test_diffcache_sketch_and_plain_scan_agree():
+    """The same prompt and decode steps through a cache that scans the 8-bit sketch and one
+    that scans the bf16 keys: identical ids, identical attention output."""
+    rng = np.random.default_rng(21)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 2, 1, 4, 16, 128, 256, 4, 8, 16, 9000
+    caches = [make_cache(L, b, seq + 32, hkv, hq, hd, budget, p, s, smax, key_sketch=ks) for ks in (True, False)]
+    scale = np.exp(rng.standard_normal((1, 1, hkv, hd))).astype(np.float32)
+    for l in range(L):
+        K = orc.f32_to_bf16(rng.standard_normal((b, seq, hkv, hd)).astype(np.float32) * scale)
+        V = rand_bf16(rng, b, seq, hkv, hd)
+        for c in caches:
+            c.prefill_update_kv_cache(dev_bf16(K), dev_bf16(V), l)
+    from diffcache_amd import _hip
+    for step in range(3):
+        for l in range(L):
+            q = dev_bf16(rand_bf16(rng, b, 1, hq * hd))
+            nk, nv = dev_bf16(rand_bf16(rng, b, 1, hkv, hd)), dev_bf16(rand_bf16(rng, b, 1, hkv, hd))
+            outs = [c.decode_attention(l, q, nk, nv, order=_hip.ORDER_BEST).clone() for c in caches]
+            assert torch.equal(caches[0].idx[l], caches[1].idx[l])
+            assert torch.equal(outs[0], outs[1])
+    # the reference-shaped hooks take the same two routes
+    for c in caches:
+        c.decode_pre_query_operation(q)
+        c.decode_query_kvcache(0)
+    assert torch.equal(caches[0].idx[0], caches[1].idx[0])
 
 
 def test_diffcache_hooks_under_graph_capture():
