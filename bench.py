@@ -26,11 +26,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one scan launch of the default workload moves, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE scaled by a known-size copy kernel (the figures and commands are kept with the
-# other profile summaries of this repository): 1 053 933 counts x 2 KiB read +
-# 12 570 counts x 1 KiB written.
-SCAN_TRAFFIC_BYTES_C3 = 1_053_933 * 2048 + 12_570 * 1024
+# HBM bytes one scan launch of config 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE scaled
+# by a known-size copy kernel (the figures and commands are kept with the other profile
+# summaries of this repository): counts x 2 KiB read + counts x 1 KiB written.
+SCAN_TRAFFIC_BYTES_C3 = {"sketch": 525_636 * 2048 + 14_044 * 1024,
+                         "bf16": 1_053_933 * 2048 + 12_570 * 1024}
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
@@ -191,13 +191,16 @@ def main() -> int:
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
-    ap.add_argument("--sketch", action="store_true",
-                    help="scan the 8-bit sketch of the keys and rescore the surviving rows exactly "
-                         "(dc_score_select_sketch_bf16 inside dc_decode_layer): same ids, half the bytes")
+    ap.add_argument("--scan", default=None, choices=["sketch", "bf16"],
+                    help="sketch (default): scan the 8-bit sketch of the keys and rescore the surviving "
+                         "rows exactly from the bf16 keys (same ids, half the bytes); bf16: stream the "
+                         "bf16 keys themselves")
     args = ap.parse_args()
-    if args.sketch and (args.dense or args.split or args.streams != 1):
-        print("bench.py: --sketch goes with the default one-call path only", file=sys.stderr)
+    other_path = args.dense or args.split or args.streams != 1
+    if args.scan == "sketch" and other_path:
+        print("bench.py: --scan sketch goes with the default one-call path only", file=sys.stderr)
         return 2
+    args.sketch = (args.scan or ("bf16" if other_path else "sketch")) == "sketch"
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
               "use --gpus 1", file=sys.stderr)
@@ -371,6 +374,8 @@ def main() -> int:
     unit_bytes = algorithmic_bytes_per_unit(region, k_eff + sink + recent, grp, hd)
     step_bytes = unit_bytes * n_units * L
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    # what the chosen path must move: the sketch scan reads hd bytes per key, not 2*hd
+    step_path_bytes = step_bytes - (n_units * L * region * hd if args.sketch else 0)
     # bytes one scan launch has to stream: the bf16 K rows, or their one-byte-per-element sketch
     score_bytes = (n_units // args.streams) * region * hd * (1 if args.sketch else 2)
     roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
@@ -378,9 +383,8 @@ def main() -> int:
                 "kernel": "sketch_prune_kernel<128>" if args.sketch else
                           "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
                 "algorithmic_bytes_per_launch": score_bytes}
-    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist" \
-            and not args.sketch:
-        roofline["traffic"] = SCAN_TRAFFIC_BYTES_C3
+    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist":
+        roofline["traffic"] = SCAN_TRAFFIC_BYTES_C3["sketch" if args.sketch else "bf16"]
     if score_ms is not None:
         ach = score_bytes / (score_ms * 1e-3) / 1e9
         roofline.update(achieved=ach, frac=ach / HBM_PEAK_GBPS, avg_launch_us=score_ms * 1e3)
@@ -404,9 +408,15 @@ def main() -> int:
                                  if args.fused else
                                  "dc_score_bf16/dc_topk_select/dc_gather_attn_bf16" if args.dense else
                                  "dc_select_state_init/dc_score_prune_bf16/dc_sparse_select/dc_gather_attn_bf16")},
+        # bytes of the reference's exact algorithm per step (every bf16 key once + the gathered
+        # K/V rows + q in/out) over the measured time.  With the sketch scan the path streams
+        # one byte per key element instead of two, so this rate can exceed the HBM peak; the
+        # bytes this call path has to move are in step_path_bytes.
         "step_hbm_gbps": step_gbps,
         "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
         "step_algorithmic_bytes": step_bytes,
+        "step_path_bytes": step_path_bytes,
+        "step_path_gbps": step_path_bytes / (ms_per_step * 1e-3) / 1e9,
         "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
         "stage_us_per_layer": stage_us,
         "roofline": roofline,
