@@ -171,8 +171,8 @@ def run_pq(args, torch, hip, dev) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS) + ["c4"])
     ap.add_argument("--mode", default="ref_dist", choices=["ref_dist", "ip"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -348,12 +348,24 @@ def main() -> int:
         step(events[-1])
     torch.cuda.synchronize()
     events = events[:-1]
+    # one more event after every step on the first micro-batch's stream: the spread of the
+    # step times (with several streams the boundaries are only approximate)
+    marks = new_events(args.steps + 1)
+    for e in marks:
+        e.record(pipes[0].stream)
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
+    marks[0].record(pipes[0].stream)
     for s in range(args.steps):
         step(events[s])
+        marks[s + 1].record(pipes[0].stream)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+    per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(args.steps))
+
+    def pct(p):
+        return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
 
     # per-kernel durations from the events of the timed region
     stage_us = None
@@ -418,6 +430,7 @@ def main() -> int:
         "step_path_bytes": step_path_bytes,
         "step_path_gbps": step_path_bytes / (ms_per_step * 1e-3) / 1e9,
         "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
+        "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
         "stage_us_per_layer": stage_us,
         "roofline": roofline,
         "setup_s": t_gen,
