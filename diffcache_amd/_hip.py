@@ -33,7 +33,7 @@ SYMBOLS = (
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
     "dc_sparse_select", "dc_score_select_bf16",
     "dc_sketch_build_bf16", "dc_sketch_select_workspace_bytes", "dc_sketch_select_state_init",
-    "dc_score_select_sketch_bf16",
+    "dc_score_select_sketch_bf16", "dc_kcheck_f32",
 )
 
 
@@ -74,7 +74,7 @@ def _load() -> C.CDLL:
         "dc_topk_select": (i, [p, i64, p, i64, i, i, i, i, i, p, p, sz, p]),
         "dc_gather_rows_bf16": (i, [p, p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, i64, i64, p]),
         "dc_attn_workspace_bytes": (sz, [i, i, i, i]),
-        "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i, i64, i,
+        "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i,
                                     i64, i64, i64, i64, i64, i64, f, p, sz, p]),
         "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, i64, i64, i64, p]),
         "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
@@ -90,6 +90,7 @@ def _load() -> C.CDLL:
         "dc_sparse_select": (i, [p, i64, i, i, i, i, i, i, p, sz, p]),
         "dc_score_select_bf16": (i, [p, p, p, i64, i, i, i, i, i64, i64, i64, i, i, i, i, p, sz, p]),
         "dc_sketch_build_bf16": (i, [p, p, p, p, i, i, i, i, i64, i64, i64, i64, i64, i64, i, p]),
+        "dc_kcheck_f32": (i, [p, i64, i, i, i, i, C.POINTER(C.c_int), i, f, p, p, p, p]),
         "dc_sketch_select_workspace_bytes": (sz, [i, i, i]),
         "dc_sketch_select_state_init": (i, [i, i, i, p, sz, p]),
         "dc_score_select_sketch_bf16": (i, [p, p, p, p, p, p, i64, i, i, i, i, i64, i64, i64, i64, i64, i64,
@@ -334,8 +335,10 @@ def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
                 n_recent: int, new_k: Optional[torch.Tensor] = None,
                 new_v: Optional[torch.Tensor] = None, scale: Optional[float] = None,
                 out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """q (b, h*group, hd) bf16 -> out (b, h*group, hd) bf16."""
+                workspace: Optional[torch.Tensor] = None,
+                n_idx_unit: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q (b, h*group, hd) bf16 -> out (b, h*group, hd) bf16.  ``n_idx_unit`` (b*h) int32:
+    per-unit number of leading ids to attend to (see ``kcheck``)."""
     ksb, ksh, ksr = _store_strides(store_k)
     vsb, vsh, vsr = _store_strides(store_v)
     b, h, _, hd = store_k.shape
@@ -353,10 +356,33 @@ def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
     _check(lib.dc_gather_attn_bf16(
         _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v"), _opt(idx, "idx"),
         _opt(new_k, "new_k"), _opt(new_v, "new_v"), _dev(out, "out"), _opt(lse, "lse"), b, h, group,
-        hd, n_idx, 0 if idx is None else idx.stride(0), region_lo, n_sink, recent_lo, n_recent,
-        ksb, ksh, ksr, vsb, vsh, vsr, scale, _dev(workspace, "workspace"), workspace.numel(),
+        hd, n_idx, 0 if idx is None else idx.stride(0), _opt(n_idx_unit, "n_idx_unit"), region_lo, n_sink,
+        recent_lo, n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, _dev(workspace, "workspace"), workspace.numel(),
         _stream()))
     return out
+
+
+def kcheck(scores: torch.Tensor, n_sel: int, hd: int, k_check_seq, attn_mass_threshold: float,
+           mode: int = MODE_REF_DIST, n_eff: Optional[torch.Tensor] = None, want_stats: bool = False):
+    """k-check of nsw.rs:198-296 on the exact, best-first scores (n_units, >= n_sel) fp32 of the
+    selected rows: n_eff (n_units) int32 = the first size of ``k_check_seq`` (below n_sel)
+    whose top rows already hold ``attn_mass_threshold`` of the estimated softmax mass, else
+    n_sel.  With ``want_stats`` also (alpha, mass), each (n_units, len(k_check_seq)) fp32."""
+    if scores.dtype != torch.float32 or scores.dim() != 2 or scores.stride(1) != 1:
+        raise DiffCacheError("scores must be a 2-d fp32 tensor with contiguous rows")
+    n_units = scores.shape[0]
+    seq = [int(x) for x in k_check_seq][:16]
+    arr = (C.c_int * max(len(seq), 1))(*seq)
+    if n_eff is None:
+        n_eff = torch.empty((n_units,), dtype=torch.int32, device=scores.device)
+    alpha = mass = None
+    if want_stats:
+        alpha = torch.empty((n_units, len(seq)), dtype=torch.float32, device=scores.device)
+        mass = torch.empty_like(alpha)
+    _check(lib.dc_kcheck_f32(_dev(scores, "scores"), scores.stride(0), n_units, n_sel, hd, mode, arr,
+                             len(seq), float(attn_mass_threshold), _dev(n_eff, "n_eff"),
+                             _opt(alpha, "alpha"), _opt(mass, "mass"), _stream()))
+    return (n_eff, alpha, mass) if want_stats else n_eff
 
 
 def append_kv(store_k: torch.Tensor, store_v: torch.Tensor, new_k: torch.Tensor,

@@ -42,8 +42,8 @@ template <int HD, int G>
 __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint32_t *__restrict__ idx, const uint16_t *__restrict__ new_k,
-    const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml, int n_h,
-    int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
+    const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml,
+    const uint32_t *__restrict__ n_idx_unit, int n_h, int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
     int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
     int64_t vsr, float scale) {
     constexpr int LPR = HD / 8;
@@ -61,13 +61,20 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const int gid = tid / LPR, col = tid % LPR;
     const int r0 = split * ROWS;
 
+    // only the first n_eff selected ids of the unit count when per-unit sizes are given
+    int n_eff = n_idx;
+    if (n_idx_unit) {
+        const uint32_t ne = n_idx_unit[unit];
+        n_eff = ne < (uint32_t)n_idx ? (int)ne : n_idx;
+    }
+
     // physical rows of this group's list positions
     uint32_t row[R];
     bool ok[R];
 #pragma unroll
     for (int t = 0; t < R; ++t) {
         const int vj = r0 + t * NG + gid;
-        ok[t] = vj < n_total;
+        ok[t] = vj < n_total && (vj < n_eff || vj >= n_idx);
         uint32_t r = 0;
         if (ok[t]) {
             if (vj < n_idx) r = (uint32_t)(region_lo + idx[(int64_t)unit * idx_stride + vj]);
@@ -301,14 +308,14 @@ AttnWs carve_attn(void *base, int n_units, int group, int hd, int n_splits) {
 template <int HD>
 int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const uint16_t *k,
                 const uint16_t *v, const uint32_t *idx, const uint16_t *new_k,
-                const uint16_t *new_v, const AttnWs &w, int n_h, int n_idx,
+                const uint16_t *new_v, const AttnWs &w, const uint32_t *n_idx_unit, int n_h, int n_idx,
                 int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
                 int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
                 int64_t vsh, int64_t vsr, float scale) {
 #define DC_ATTN_CASE(GG)                                                                           \
     case GG:                                                                                       \
         hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, q, k, v, idx, \
-                           new_k, new_v, w.acc, w.ml, n_h, n_idx, idx_stride,                      \
+                           new_k, new_v, w.acc, w.ml, n_idx_unit, n_h, n_idx, idx_stride,                      \
                            region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, ksb, ksh,    \
                            ksr, vsb, vsh, vsr, scale);                                             \
         return 0;
@@ -336,7 +343,8 @@ extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_
 extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
                                    const void *new_k, const void *new_v, void *out, float *lse,
                                    int n_b, int n_h, int group, int hd, int n_idx,
-                                   int64_t idx_unit_stride, int64_t region_lo, int n_sink,
+                                   int64_t idx_unit_stride, const uint32_t *n_idx_unit,
+                                   int64_t region_lo, int n_sink,
                                    int64_t recent_lo, int n_recent, int64_t ksb, int64_t ksh,
                                    int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
                                    void *workspace, size_t workspace_bytes, void *stream) {
@@ -376,15 +384,15 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
     const uint16_t *nk16 = (const uint16_t *)new_k, *nv16 = (const uint16_t *)new_v;
     uint16_t *o16 = (uint16_t *)out;
     if (hd == 64)
-        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else if (hd == 128)
-        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                               plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else
-        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_h, n_idx,
+        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                               plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     DC_REQUIRE(rc == 0, "dc_gather_attn_bf16: unsupported group %d", group);

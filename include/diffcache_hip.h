@@ -200,6 +200,9 @@ size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attend
  * q, out: (n_b, n_h*group, hd) bf16, query head h*group + g belongs to kv-head h.
  * out = softmax(q . K^T * scale) . V, fp32 softmax and accumulation, bf16 out;
  * lse (n_b, n_h*group) fp32 log-sum-exp of the scaled logits, or NULL.
+ * n_idx_unit: NULL, or (n_b*n_h) uint32: unit u attends only to its first
+ * min(n_idx_unit[u], n_idx) retrieved rows (the output of dc_kcheck_f32 on ids in
+ * DC_ORDER_BEST order); the always-kept rows are unaffected.
  * Replaces flash_attn_with_kvcache over the assembled buffer
  * (src/diffcache/base.py:134-142) and the buffer assembly it reads
  * (src/diffcache/kvcache/diffcache.py:48-66,186-209).
@@ -207,10 +210,30 @@ size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attend
 int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
                         const void *new_k, const void *new_v, void *out, float *lse, int n_b,
                         int n_h, int group, int hd, int n_idx, int64_t idx_unit_stride,
-                        int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-                        int64_t k_batch_stride, int64_t k_head_stride, int64_t k_row_stride,
-                        int64_t v_batch_stride, int64_t v_head_stride, int64_t v_row_stride,
-                        float scale, void *workspace, size_t workspace_bytes, void *stream);
+                        const uint32_t *n_idx_unit, int64_t region_lo, int n_sink, int64_t recent_lo,
+                        int n_recent, int64_t k_batch_stride, int64_t k_head_stride,
+                        int64_t k_row_stride, int64_t v_batch_stride, int64_t v_head_stride,
+                        int64_t v_row_stride, float scale, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
+/*
+ * k-check (diffcache_cpu/src/nsw.rs:198-296): how many of a unit's best rows are
+ * worth attending to.  scores (n_units, scores_unit_stride) fp32: the exact scores of
+ * the n_sel selected rows, best first (dc_score_gathered_bf16 on ids in DC_ORDER_BEST
+ * order).  The logit of a row is (65536 - f32(65536 - score)) / sqrt(hd) as in
+ * nsw.rs:282-286 (score / sqrt(hd) in DC_MODE_IP).  For each size H of k_check_seq
+ * (a host array of at most 16 ints), in order, while H < n_sel: a power law is
+ * fitted to the logits of ranks 5..H (nsw.rs:198-241), the share of the softmax mass
+ * held by the top H is estimated (nsw.rs:243-278), and the first H whose share
+ * reaches attn_mass_threshold is written to n_eff[u]; if none does, n_eff[u] = n_sel.
+ * alpha_out, mass_out: NULL or (n_units, n_seq) fp32, NaN where a size was not
+ * evaluated or the reference returns None.  The reference only reports the outcome
+ * of the check (nsw.rs:367-379); feeding n_eff to dc_gather_attn_bf16 is what acts
+ * on it.
+ */
+int dc_kcheck_f32(const float *scores, int64_t scores_unit_stride, int n_units, int n_sel, int hd,
+                  int mode, const int *k_check_seq, int n_seq, float attn_mass_threshold,
+                  uint32_t *n_eff, float *alpha_out, float *mass_out, void *stream);
 
 /*
  * Append one token: k_store[b, h, pos, :] = new_k[b, h, :] (same for v).

@@ -26,6 +26,11 @@ assemble_kvbuf         src/diffcache/kvcache/diffcache.py:48-66,186-209
 sparse_attention       src/diffcache/base.py:134-142 (flash-attn decode call,
                        default scale 1/sqrt(hd), new token appended)
 decode_layer           src/diffcache/base.py:150-155 call order
+fit_alpha_from_logits  diffcache_cpu/src/nsw.rs:198-241
+estimate_top_h_mass    diffcache_cpu/src/nsw.rs:243-278
+k_check_early_stoppable diffcache_cpu/src/nsw.rs:280-296
+k_check_budget         the epoch loop of nsw.rs:302-303,339,367-379 applied to
+                       the exact, sorted result list
 pq_*                   no reference source (evaluation/impl/pqcache is an
                        empty directory): PARITY UNPINNED at the reference;
                        pinned by closed forms in tests/test_oracle_pq.py
@@ -450,6 +455,96 @@ def pq_search(q_u16: np.ndarray, k_u16: np.ndarray, codes: np.ndarray, lut_f32: 
     packed = (key32(exact, MODE_IP).astype(np.uint64) << np.uint64(32)) | cand.astype(np.uint64)
     packed = np.sort(packed)[:min(k, len(cand))]
     return cand, (packed & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+
+
+# --------------------------------------------------------------------------
+# k-check: does the top-H already hold the wanted attention mass?
+# (nsw.rs:198-296; no tests in the reference -- pinned by closed forms in
+# tests/test_oracle_kcheck.py)
+# --------------------------------------------------------------------------
+
+K_CHECK_MIN_RANK = 5  # nsw.rs:288
+
+
+def fit_alpha_from_logits(logits_sorted: np.ndarray, min_rank: int) -> Optional[np.float32]:
+    """Least-squares slope of logit against ln(rank) over ranks min_rank..H; alpha = -slope
+    (nsw.rs:198-241).  Sums in f64 in rank order, result cast to f32."""
+    z = np.asarray(logits_sorted, dtype=np.float32)
+    h = len(z)
+    if h == 0 or min_rank == 0 or min_rank >= h:
+        return None
+    n = float(h - min_rank + 1)
+    if n < 2.0:
+        return None
+    sx = sy = sxx = sxy = 0.0
+    for idx in range(min_rank - 1, h):
+        x = float(np.log(np.float64(idx + 1)))
+        y = float(z[idx])
+        sx += x
+        sy += y
+        sxx += x * x
+        sxy += x * y
+    denom = n * sxx - sx * sx
+    if abs(denom) < 1e-12:
+        return None
+    b = (n * sxy - sx * sy) / denom
+    return np.float32(-b)
+
+
+def estimate_top_h_mass(logits_sorted: np.ndarray, h: int, alpha: np.float32) -> Optional[np.float32]:
+    """Share of the softmax mass the first h logits hold when the rest follows a power law
+    with exponent alpha: head / (head + v_h * h / (alpha - 1)), all in f32, sums in rank
+    order (nsw.rs:243-278)."""
+    z = np.asarray(logits_sorted, dtype=np.float32)
+    if h == 0 or h > len(z):
+        return None
+    alpha = np.float32(alpha)
+    if alpha <= np.float32(1.0):
+        return None
+    head = z[:h]
+    mx = np.float32(head.max())
+    head_sum = np.float32(0.0)
+    for v in head:
+        head_sum = np.float32(head_sum + np.exp(np.float32(v - mx), dtype=np.float32))
+    v_h = np.exp(np.float32(head[h - 1] - mx), dtype=np.float32)
+    tail = np.float32(np.float32(v_h * np.float32(h)) / np.float32(alpha - np.float32(1.0)))
+    denom = np.float32(head_sum + tail)
+    if denom <= 0:
+        return None
+    return np.float32(head_sum / denom)
+
+
+def k_check_logits(dists: np.ndarray, dim: int) -> np.ndarray:
+    """(65536 - dist) / sqrt(dim) in f32 (nsw.rs:282-286)."""
+    d = np.asarray(dists, dtype=np.float32)
+    return ((np.float32(65536.0) - d) / np.float32(np.sqrt(np.float32(dim)))).astype(np.float32)
+
+
+def k_check_early_stoppable(dists_sorted: np.ndarray, dim: int, attn_mass_threshold: float) -> bool:
+    """nsw.rs:280-296 on the ascending distances of the current best H."""
+    logits = k_check_logits(dists_sorted, dim)
+    alpha = fit_alpha_from_logits(logits, K_CHECK_MIN_RANK)
+    if alpha is None:
+        return False
+    mass = estimate_top_h_mass(logits, len(logits), alpha)
+    if mass is None:
+        return False
+    return bool(mass >= np.float32(attn_mass_threshold))
+
+
+def k_check_budget(dists_sorted: np.ndarray, dim: int, k_check_seq: Sequence[int],
+                   attn_mass_threshold: float) -> int:
+    """The number of best rows worth attending to: the first H of k_check_seq (H < ef, taken
+    in order, nsw.rs:302-303,377-378) whose top-H passes the k-check, else ef = len(dists).
+    The reference runs this inside its graph search on the H best found so far; on the exact,
+    complete result list those are the first H entries."""
+    ef = len(dists_sorted)
+    for h in k_check_seq:
+        if h >= ef:
+            break
+        if k_check_early_stoppable(np.asarray(dists_sorted)[:h], dim, attn_mass_threshold):
+            return int(h)
+    return ef
 
 
 # --------------------------------------------------------------------------

@@ -470,6 +470,87 @@ def test_gather_attention_matches_float64(hd, g, n_idx, n_sink, n_recent, new_to
             assert np.allclose(lse[bi, hi * g:(hi + 1) * g], wl, rtol=1e-4, atol=1e-4)
 
 
+def test_gather_attention_with_per_unit_counts():
+    # every unit attends to its own number of leading ids (whole splits drop out for some)
+    rng = np.random.default_rng(91)
+    b, h, g, hd, n_idx, n_sink, n_recent = 2, 2, 4, 128, 700, 4, 20
+    n_ctx = n_sink + n_recent + 3000
+    region_lo, recent_lo = n_sink, n_ctx - n_recent
+    k, v = rand_bf16(rng, b, h, n_ctx, hd), rand_bf16(rng, b, h, n_ctx, hd)
+    q = rand_bf16(rng, b, h * g, hd, scale=1.5)
+    idx = np.stack([rng.choice(recent_lo - region_lo, n_idx, replace=False) for _ in range(b * h)]
+                   ).astype(np.int32)
+    nk, nv = rand_bf16(rng, b, h, hd), rand_bf16(rng, b, h, hd)
+    counts = np.int32([700, 1, 130, 0])
+    out = hip.gather_attn(to_dev_bf16(q), to_dev_bf16(k), to_dev_bf16(v), torch.from_numpy(idx).to(DEV),
+                          n_idx, region_lo, n_sink, recent_lo, n_recent, to_dev_bf16(nk), to_dev_bf16(nv),
+                          n_idx_unit=torch.from_numpy(counts).to(DEV))
+    got = orc.bf16_to_f32(to_np_u16(out))
+    for bi in range(b):
+        for hi in range(h):
+            u = bi * h + hi
+            rows = orc.attended_rows(idx[u, :counts[u]].astype(np.uint32), region_lo, recent_lo, n_ctx)
+            want, _ = orc.sparse_attention(q[bi, hi * g:(hi + 1) * g], k[bi, hi][rows], v[bi, hi][rows],
+                                           nk[bi, hi], nv[bi, hi])
+            assert bf16_close(got[bi, hi * g:(hi + 1) * g], want)
+
+
+def kcheck_case(scores_sorted, hd, seq, thr, mode):
+    """GPU k-check against the oracle on best-first scores (n_units, n_sel)."""
+    n_units, n_sel = scores_sorted.shape
+    n_eff, alpha, mass = hip.kcheck(torch.from_numpy(scores_sorted).to(DEV), n_sel, hd, seq, thr, mode,
+                                    want_stats=True)
+    n_eff, alpha, mass = n_eff.cpu().numpy(), alpha.cpu().numpy(), mass.cpu().numpy()
+    for u in range(n_units):
+        s = scores_sorted[u]
+        d = orc.ref_dist(s) if mode == orc.MODE_REF_DIST else (np.float32(65536.0) - s).astype(np.float32)
+        # in DC_MODE_IP the logits are score / sqrt(hd): feed the oracle distances that give them
+        logits = orc.k_check_logits(d, hd) if mode == orc.MODE_REF_DIST else (s / np.float32(np.sqrt(np.float32(hd)))).astype(np.float32)
+        want_eff, borderline = n_sel, False
+        for e, hh in enumerate(seq):
+            if hh >= n_sel:
+                break
+            a = orc.fit_alpha_from_logits(logits[:hh], orc.K_CHECK_MIN_RANK)
+            if a is None:
+                assert np.isnan(alpha[u, e])
+                continue
+            assert abs(float(alpha[u, e]) - float(a)) <= 2e-5 * max(1.0, abs(float(a))), (u, e)
+            m = orc.estimate_top_h_mass(logits[:hh], hh, a)
+            if m is None:
+                assert np.isnan(mass[u, e])
+                continue
+            # the reference sums exp() sequentially in f32; the kernel sums the same f32 terms in
+            # f64: they agree to the rounding of an H-term f32 sum
+            assert abs(float(mass[u, e]) - float(m)) <= 2e-4, (u, e, mass[u, e], m)
+            if abs(float(m) - thr) <= 2e-4:
+                borderline = True
+                break
+            if float(m) >= thr:
+                want_eff = hh
+                break
+        if not borderline:
+            assert int(n_eff[u]) == want_eff, (u, n_eff[u], want_eff)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_kcheck_matches_oracle(mode):
+    rng = np.random.default_rng(5 + mode)
+    hd, n_sel = 128, 2048
+    sq = np.sqrt(np.float32(hd))
+    r = np.arange(1, n_sel + 1, dtype=np.float64)
+    rows = []
+    for alpha, noise in [(3.0, 0.0), (1.6, 0.05), (1.05, 0.02), (0.5, 0.1), (2.2, 0.3)]:
+        z = 12.0 - alpha * np.log(r) + noise * rng.standard_normal(n_sel)
+        rows.append(np.sort((z * sq).astype(np.float32))[::-1])
+    rows.append(np.full(n_sel, 7.5, np.float32))                      # flat: alpha = 0, never stoppable
+    rows.append(np.sort((rng.standard_normal(n_sel) * 30).astype(np.float32))[::-1])
+    scores = np.ascontiguousarray(np.stack(rows))
+    seq = [100, 200, 300, 400, 800, 1600, 3200, 6400, 12800, 25600]   # the reference's default
+    for thr in (0.5, 0.9, 0.99):
+        kcheck_case(scores, hd, seq, thr, mode)
+    kcheck_case(scores[:, :150], 64, [3, 5, 6, 100, 150, 200], 0.7, mode)   # sizes <= 5 and >= n_sel
+
+
 def test_attention_identities_on_gpu():
     rng = np.random.default_rng(33)
     b, h, g, hd, n = 1, 2, 4, 128, 2500
