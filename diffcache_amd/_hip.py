@@ -496,13 +496,14 @@ def pq_adc_scan(codes: torch.Tensor, lut: torch.Tensor, hist: Optional[torch.Ten
     return scores
 
 
-def score_gathered(store_k: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, row_offset: int = 0
-                   ) -> torch.Tensor:
+def score_gathered(store_k: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, row_offset: int = 0,
+                   scores: Optional[torch.Tensor] = None) -> torch.Tensor:
     sb, sh, sr = _store_strides(store_k)
     b, h, _, hd = store_k.shape
     q = q.contiguous()
     n_idx = idx.shape[1]
-    scores = torch.empty((b * h, n_idx), dtype=torch.float32, device=q.device)
+    if scores is None:
+        scores = torch.empty((b * h, n_idx), dtype=torch.float32, device=q.device)
     _check(lib.dc_score_gathered_bf16(_dev(store_k, "store_k"), _dev(q, "q"), _dev(idx, "idx"),
                                       _dev(scores, "scores"), b, h, n_idx, idx.stride(0), hd, row_offset,
                                       sb, sh, sr, scores.stride(0), _stream()))

@@ -58,6 +58,7 @@ class DiffCache:
         key_mode: str = "ref_dist",
         device: str = "cuda",
         key_sketch: bool = True,
+        use_k_check: bool = False,
     ) -> None:
         self.num_layers = num_layers
         self.batch_size = batch_size
@@ -119,6 +120,14 @@ class DiffCache:
         self._ws_ready = False        # a decode_attention call has left its select state ready
         self._hook_ws_ready = False   # a decode_query_kvcache call (sketch route) has
         self._attn_out: Optional[torch.Tensor] = None
+        # k-check (nsw.rs:198-296): with use_k_check, decode_attention attends only to the
+        # leading rows of each unit's best-first list that the check finds sufficient
+        # (attn_mass_threshold, k_check_seq); n_eff[layer] holds the sizes it chose.
+        self.use_k_check = use_k_check
+        self.n_eff = [torch.zeros((n_units,), device=self.device, dtype=torch.int32)
+                      for _ in range(num_layers)] if use_k_check else []
+        self._kc_scores: Optional[torch.Tensor] = None
+        self._attn_ws: Optional[torch.Tensor] = None
         self._prefix0 = kvbuf_prefix_len
         self._suffix0 = kvbuf_suffix_len
 
@@ -258,6 +267,11 @@ class DiffCache:
                 self._attn_out = torch.empty((b, hq, hd), device=self.device, dtype=torch.bfloat16)
             out = self._attn_out
         ws = self._ensure_workspace()
+        if self.use_k_check and min(hi - lo, self.retrieval_budget) > 0:
+            self._decode_attention_k_check(layer_idx, q, out, ws)
+            if layer_idx == self.num_layers - 1:
+                self.kvbuf_suffix_len += 1
+            return out
         hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
                          self.kvbuf_suffix_len + 1, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
                          mode=self.mode, order=order, select_state_ready=self._ws_ready,
@@ -267,6 +281,38 @@ class DiffCache:
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
         return out
+
+    def _decode_attention_k_check(self, layer_idx: int, q: torch.Tensor, out: torch.Tensor,
+                                  ws: torch.Tensor) -> None:
+        """select (best first) -> exact scores of the selected rows -> k-check -> attention over
+        the leading n_eff rows of every unit plus the always-kept rows."""
+        lo, hi = self._region()
+        n_sel = min(hi - lo, self.retrieval_budget)
+        n_units = self.batch_size * self.num_kv_heads
+        ks, vs, idx = self.kstore[layer_idx], self.vstore[layer_idx], self.idx[layer_idx]
+        if self.key_sketch:
+            hip.score_select_sketch(ks, self.sketch[layer_idx], q, lo, hi - lo, n_sel, self.mode,
+                                    hip.ORDER_BEST, q_group=self.group, idx_out=idx, workspace=ws,
+                                    state_ready=self._hook_ws_ready)
+            self._hook_ws_ready = True
+        else:
+            hip.score_select(ks, q, lo, hi - lo, n_sel, self.mode, hip.ORDER_BEST, q_group=self.group,
+                             idx_out=idx, workspace=ws)
+            self._hook_ws_ready = False
+        self._ws_ready = False
+        hip.group_mean(q, self.group, out=self.qbuf.view(-1, self.head_dim), hd=self.head_dim)
+        if self._kc_scores is None or self._kc_scores.shape[1] != n_sel:
+            self._kc_scores = torch.empty((n_units, n_sel), device=self.device, dtype=torch.float32)
+        hip.score_gathered(ks, self.qbuf, idx[:, :n_sel], row_offset=lo, scores=self._kc_scores)
+        hip.kcheck(self._kc_scores, n_sel, self.head_dim, self.k_check_seq, self.attn_mass_threshold,
+                   self.mode, n_eff=self.n_eff[layer_idx])
+        n_recent = self.kvbuf_suffix_len + 1
+        need = hip.lib.dc_attn_workspace_bytes(n_units, self.group, self.head_dim,
+                                               n_sel + self.kvbuf_prefix_len + self.kvbuf_suffix_maxlen + 1)
+        if self._attn_ws is None or self._attn_ws.numel() < need:
+            self._attn_ws = hip.alloc_workspace(need, self.device)
+        hip.gather_attn(q, ks, vs, idx, n_sel, lo, lo, hi, n_recent, out=out, workspace=self._attn_ws,
+                        n_idx_unit=self.n_eff[layer_idx])
 
     # ------------------------------------------------------------------ prefill cache
     def save_prefill_cache(self, prefill_cache_path: str) -> None:

@@ -158,8 +158,16 @@ def test_data_layer_save_load_roundtrip(tmp_path):
 # ---------------------------------------------------------------- DiffCache
 
 def make_cache(num_layers, b, max_len, hkv, hq, hd, budget, p, s, smax, key_mode="ref_dist",
-               key_sketch=True):
+               key_sketch=True, **extra):
     from diffcache_amd import DiffCache
+    if extra:
+        kw = dict(num_layers=num_layers, batch_size=b, max_length=max_len, num_kv_heads=hkv,
+                  num_q_heads=hq, head_dim=hd, retrieval_budget=budget, nsw_m=16, nsw_ef_cons=200,
+                  kvbuf_prefix_len=p, kvbuf_suffix_len=s, kvbuf_suffix_maxlen=smax,
+                  attn_mass_threshold=0.9, k_check_seq=[1048576],
+                  r_sq=[[4.0] * hkv for _ in range(num_layers)], key_mode=key_mode, key_sketch=key_sketch)
+        kw.update(extra)
+        return DiffCache(**kw)
     return DiffCache(key_sketch=key_sketch, num_layers=num_layers, batch_size=b, max_length=max_len, num_kv_heads=hkv,
                      num_q_heads=hq, head_dim=hd, retrieval_budget=budget, nsw_m=16, nsw_ef_cons=200,
                      kvbuf_prefix_len=p, kvbuf_suffix_len=s, kvbuf_suffix_maxlen=smax,
@@ -272,6 +280,53 @@ def test_diffcache_sketch_and_plain_scan_agree():
         c.decode_pre_query_operation(q)
         c.decode_query_kvcache(0)
     assert torch.equal(caches[0].idx[0], caches[1].idx[0])
+
+
+def test_diffcache_decode_attention_with_k_check():
+    """use_k_check: every unit attends to the leading rows the check of nsw.rs:198-296 finds
+    sufficient.  One kv-head sees keys whose scores fall off fast (few rows suffice), the other
+    near-uniform scores (the whole budget is kept)."""
+    rng = np.random.default_rng(44)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 1, 1, 2, 4, 128, 512, 4, 8, 16, 6000
+    kseq, thr = [16, 32, 64, 128, 256], 0.9
+    cache = make_cache(L, b, seq + 32, hkv, hq, hd, budget, p, s, smax, use_k_check=True,
+                       k_check_seq=kseq, attn_mass_threshold=thr)
+    q = rand_bf16(rng, b, 1, hq * hd)
+    qf = orc.bf16_to_f32(q).reshape(b, hq, hd)
+    qmean = orc.bf16_to_f32(orc.group_mean_bf16(q.reshape(b, hq, hd), hkv))          # (b, hkv, hd)
+    K = orc.bf16_to_f32(rand_bf16(rng, b, seq, hkv, hd, scale=0.2))
+    # head 0: 300 keys aligned with the mean query, with strengths that decay like a power law
+    u0 = qmean[0, 0] / np.linalg.norm(qmean[0, 0])
+    pos = rng.choice(np.arange(p, seq - s), 300, replace=False)
+    strength = 200.0 - 30.0 * np.log(np.arange(1, 301))
+    K[0, pos, 0, :] += (strength[:, None] / np.linalg.norm(qmean[0, 0])) * u0[None, :]
+    K = orc.f32_to_bf16(K)
+    V = rand_bf16(rng, b, seq, hkv, hd)
+    cache.prefill_update_kv_cache(dev_bf16(K), dev_bf16(V), 0)
+    nk, nv = rand_bf16(rng, b, 1, hkv, hd), rand_bf16(rng, b, 1, hkv, hd)
+    out = cache.decode_attention(0, dev_bf16(q), dev_bf16(nk), dev_bf16(nv))
+    torch.cuda.synchronize()
+    got = orc.bf16_to_f32(np_u16(out))
+    from diffcache_amd import _hip
+    p_len, s_len, lo, hi = orc.region_split(seq, p, s)
+    ids = cache.idx[0].cpu().numpy().astype(np.uint32)
+    n_eff = cache.n_eff[0].cpu().numpy()
+    kk = np.transpose(K, (0, 2, 1, 3))[0]                                             # (hkv, n, hd)
+    vv = np.transpose(V, (0, 2, 1, 3))[0]
+    sc = _hip.score(cache.kstore[0], dev_bf16(orc.group_mean_bf16(q.reshape(b, hq, hd), hkv)), lo, hi - lo,
+                    _hip.MODE_REF_DIST).cpu().numpy()
+    g = hq // hkv
+    for h in range(hkv):
+        want_ids = orc.topk_select(sc[h], budget, orc.MODE_REF_DIST)
+        assert np.array_equal(ids[h, :budget], want_ids)
+        d = orc.ref_dist(sc[h][want_ids])
+        want_eff = orc.k_check_budget(d, hd, kseq, thr)
+        assert int(n_eff[h]) == want_eff, (h, n_eff[h], want_eff)
+        rows = orc.attended_rows(want_ids[:want_eff], lo, hi, seq)
+        want, _ = orc.sparse_attention(q.reshape(b, hq, hd)[0, h * g:(h + 1) * g], kk[h][rows], vv[h][rows],
+                                       nk[0, 0, h], nv[0, 0, h])
+        assert bf16_close(got[0, h * g:(h + 1) * g], want)
+    assert n_eff[0] < budget and n_eff[1] == budget
 
 
 def test_diffcache_hooks_under_graph_capture():
