@@ -52,21 +52,45 @@ def algorithmic_bytes_per_unit(n_region: int, attended: int, group: int, hd: int
 
 def make_layer(torch, cfg, layer: int, cfg_id: int, dev, k, v):
     """Synthetic K, V, q, new k/v of one layer, generated on the device into the
-    layer's views k, v of the store."""
+    layer's views k, v of the store.  Seed = 1000 * config + layer.
+    config 2: keys N(0,1) x per-channel log-normal scale, queries N(0,1);
+    config 3: the same keys, queries 0.7 * mean of a random 32-key cluster + 0.3 * N(0,1);
+    config 5: keys in 256 Gaussian clusters (centres N(0,1), std 0.1), every query head
+              aimed at the mean of 1-4 cluster centres."""
     g = torch.Generator(device=dev).manual_seed(1000 * cfg_id + layer)
     b, hkv, hq, hd, n = cfg["batch"], cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"]
-    k.normal_(generator=g)
-    v.normal_(generator=g)
-    # per-channel log-normal scale (sigma 1), one vector per kv head: outlier channels
-    scale = torch.exp(torch.randn((1, hkv, 1, hd), generator=g, device=dev)).to(torch.bfloat16)
-    k.mul_(scale)
-    # queries: 0.7 * mean of a random 32-key cluster + 0.3 * N(0,1), per query head
     grp = hq // hkv
-    pick = torch.randint(0, n, (b, hq, 32), generator=g, device=dev)
-    bi = torch.arange(b, device=dev).view(b, 1, 1).expand(b, hq, 32)
-    hi = (torch.arange(hq, device=dev) // grp).view(1, hq, 1).expand(b, hq, 32)
-    centre = k[bi, hi, pick].float().mean(dim=2)
-    q = (0.7 * centre + 0.3 * torch.randn((b, hq, hd), generator=g, device=dev)).to(torch.bfloat16)
+    v.normal_(generator=g)
+    if cfg_id == 5:
+        n_cl = 256
+        centres = torch.randn((b, hkv, n_cl, hd), generator=g, device=dev)
+        k.normal_(generator=g)
+        k.mul_(0.1)
+        member = torch.randint(0, n_cl, (b, hkv, n), generator=g, device=dev)
+        for bi in range(b):
+            for hi in range(hkv):     # one unit at a time: 256 MB of fp32 centres per gather
+                k[bi, hi].add_(centres[bi, hi][member[bi, hi]].to(torch.bfloat16))
+        n_t = torch.randint(1, 5, (b, hq), generator=g, device=dev)
+        pick = torch.randint(0, n_cl, (b, hq, 4), generator=g, device=dev)
+        use = (torch.arange(4, device=dev).view(1, 1, 4) < n_t.unsqueeze(-1)).float()
+        bi = torch.arange(b, device=dev).view(b, 1, 1).expand(b, hq, 4)
+        hi = (torch.arange(hq, device=dev) // grp).view(1, hq, 1).expand(b, hq, 4)
+        target = (centres[bi, hi, pick] * use.unsqueeze(-1)).sum(2) / n_t.unsqueeze(-1).float()
+        q = (target + 0.1 * torch.randn((b, hq, hd), generator=g, device=dev)).to(torch.bfloat16)
+    else:
+        k.normal_(generator=g)
+        # per-channel log-normal scale (sigma 1), one vector per kv head: outlier channels
+        scale = torch.exp(torch.randn((1, hkv, 1, hd), generator=g, device=dev)).to(torch.bfloat16)
+        k.mul_(scale)
+        if cfg_id == 2:
+            q = torch.randn((b, hq, hd), generator=g, device=dev).to(torch.bfloat16)
+        else:
+            # queries: 0.7 * mean of a random 32-key cluster + 0.3 * N(0,1), per query head
+            pick = torch.randint(0, n, (b, hq, 32), generator=g, device=dev)
+            bi = torch.arange(b, device=dev).view(b, 1, 1).expand(b, hq, 32)
+            hi = (torch.arange(hq, device=dev) // grp).view(1, hq, 1).expand(b, hq, 32)
+            centre = k[bi, hi, pick].float().mean(dim=2)
+            q = (0.7 * centre + 0.3 * torch.randn((b, hq, hd), generator=g, device=dev)).to(torch.bfloat16)
     new_k = torch.randn((b, hkv, hd), generator=g, device=dev).to(torch.bfloat16)
     new_v = torch.randn((b, hkv, hd), generator=g, device=dev).to(torch.bfloat16)
     return k, v, q.contiguous(), new_k, new_v
