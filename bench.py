@@ -215,6 +215,9 @@ def main() -> int:
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture one decode step (all layers) in a HIP graph and time its replays; "
+                         "reported as graph_step_us next to the eager figure")
     ap.add_argument("--scan", default=None, choices=["sketch", "bf16"],
                     help="sketch (default): scan the 8-bit sketch of the keys and rescore the surviving "
                          "rows exactly from the bf16 keys (same ids, half the bytes); bf16: stream the "
@@ -391,6 +394,25 @@ def main() -> int:
     def pct(p):
         return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
 
+    graph_step_us = None
+    if args.graph and args.streams == 1 and args.fused:
+        # every call of the step only enqueues kernels on the stream, so the whole step can be
+        # captured; the select state is already "left ready" by the eager steps above
+        cap_stream = pipes[0].stream
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=cap_stream):
+            for l in range(L):
+                pipes[0].layer(l, None)
+        torch.cuda.synchronize()
+        for _ in range(max(args.warmup, 1)):
+            graph.replay()
+        torch.cuda.synchronize()
+        tg = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_step_us = (time.perf_counter() - tg) * 1e6 / args.steps
+
     # per-kernel durations from the events of the timed region
     stage_us = None
     score_ms = None
@@ -455,6 +477,7 @@ def main() -> int:
         "step_path_gbps": step_path_bytes / (ms_per_step * 1e-3) / 1e9,
         "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
         "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
+        "graph_step_us": graph_step_us,
         "stage_us_per_layer": stage_us,
         "roofline": roofline,
         "setup_s": t_gen,

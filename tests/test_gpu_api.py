@@ -371,6 +371,47 @@ def test_diffcache_hooks_under_graph_capture():
         (torch.randn(1000, device=DEV) * 2).sum().item()    # unrelated eager work between replays
 
 
+@pytest.mark.parametrize("with_sketch", [True, False])
+def test_decode_layer_chain_in_a_graph(with_sketch):
+    """The whole per-layer chain (scan, select, attention) captured in one HIP graph: every
+    replay, with fresh queries and eager work and synchronisations in between, must equal the
+    eager call."""
+    from diffcache_amd import _hip
+    rng = np.random.default_rng(31)
+    b, hkv, hq, hd, n, budget, p, s = 1, 4, 16, 128, 20000, 512, 4, 32
+    k, v = dev_bf16(rand_bf16(rng, b, hkv, n, hd)), dev_bf16(rand_bf16(rng, b, hkv, n, hd))
+    lo, hi = p, n - s
+    sk = _hip.Sketch(k).build(k, lo, hi - lo) if with_sketch else None
+    ws = _hip.alloc_workspace(_hip.layer_workspace_bytes(b * hkv, hi - lo, budget, hq // hkv, hd,
+                                                        budget + p + s + 1), DEV)
+    q_static = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    nk, nv = dev_bf16(rand_bf16(rng, b, hkv, hd)), dev_bf16(rand_bf16(rng, b, hkv, hd))
+    idx_g = torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV)
+    out_g = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    idx_e, out_e = torch.zeros_like(idx_g), torch.zeros_like(out_g)
+
+    def call(idx, out, ready):
+        _hip.decode_layer(q_static, k, v, lo, hi, s, budget, None, idx, out, ws, nk, nv,
+                          order=_hip.ORDER_INDEX, select_state_ready=ready, sketch=sk)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(idx_e, out_e, False)          # warm-up; leaves the select state ready
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(idx_g, out_g, True)
+    for it in range(4):
+        q_static.copy_(dev_bf16(rand_bf16(rng, b, hq, hd)))
+        g.replay()
+        torch.cuda.synchronize()
+        call(idx_e, out_e, True)
+        torch.cuda.synchronize()
+        assert torch.equal(idx_g, idx_e) and torch.equal(out_g, out_e), it
+        (torch.randn(1000, device=DEV) * 2).sum().item()    # unrelated eager work between replays
+
+
 def test_diffcache_prefill_cache_roundtrip(tmp_path):
     rng = np.random.default_rng(40)
     L, b, hkv, hq, hd, budget, p, s, smax, seq = 2, 1, 2, 4, 64, 32, 4, 8, 16, 300
