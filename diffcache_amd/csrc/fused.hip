@@ -22,6 +22,12 @@
 // from the complete histogram and splits the survivors into certain members and
 // candidates; select_finish_kernel (one block per unit) finishes with the same
 // radix select as finalize_kernel.
+//
+// The sketch route reads half the bytes for the same result: sketch_prune_kernel
+// is the same scan over an 8-bit sketch of the keys (one byte per element, see
+// sketch.hip) with a margin that makes its pruning safe, rescore_kernel computes
+// the exact scores of the rows that survive it and lists them as candidates, and
+// select_finish_kernel picks the k best of that list.
 #include "dc_common.h"
 #include "dc_select.h"
 
@@ -32,7 +38,7 @@ constexpr int kRowsPerBlockStep = 256;
 constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
-constexpr int kCandLds = 8192;
+constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
 constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
 static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kThreads == DC_HIST_BINS, "bin split");
 
