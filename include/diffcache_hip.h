@@ -287,8 +287,8 @@ typedef struct dc_layer_args {
     int select_state_ready; /* streaming select only (scores == NULL).  0: the workspace is
                              initialised first.  1: the caller vouches that the last call on this
                              workspace was a dc_decode_layer with the same n_b, n_h, region length
-                             and budget and scores == NULL, which leaves the select state ready;
-                             the init kernel is skipped */
+                             and budget and scores == NULL (with or without a sketch), which
+                             leaves the select state ready; the init kernel is skipped */
     void *ev_scan_begin;  /* optional hipEvent_t pair recorded on `stream` right before and */
     void *ev_scan_end;    /* right after the scan kernel (for timing it in place), or NULL */
     const uint8_t *sketch_codes; /* NULL, or the sketch of the K store (row 0 = store row 0): the
