@@ -353,6 +353,44 @@ def test_sketch_select_matches_dense_path(mode, hd, n_rows, budget):
     check_sketch(k, q, lo, n_rows, budget, mode, hip.ORDER_ANY)
 
 
+@pytest.mark.parametrize("law", ["heavy_tail", "tiny", "huge", "sparse", "one_hot_query", "constant_rows",
+                                 "sorted_scores", "negative_scores"])
+def test_sketch_select_is_exact_on_awkward_data(law):
+    """Whatever the data do to the sketch's fit, the ids are those of the exact scan."""
+    rng = np.random.default_rng(sum(map(ord, law)))
+    b, h, n, hd, budget = 1, 2, 24000, 128, 700
+    kf = rng.standard_normal((b, h, n, hd)).astype(np.float32)
+    qf = rng.standard_normal((b, h, hd)).astype(np.float32)
+    if law == "heavy_tail":            # Cauchy keys: a few huge elements set the scales
+        kf = rng.standard_cauchy((b, h, n, hd)).astype(np.float32)
+    elif law == "tiny":
+        kf *= 1e-20
+        qf *= 1e-10
+    elif law == "huge":
+        kf *= 1e15
+        qf *= 1e10
+    elif law == "sparse":              # 95 % zeros
+        kf *= (rng.random((b, h, n, hd)) < 0.05)
+    elif law == "one_hot_query":       # the score is one key column
+        qf[:] = 0
+        qf[0, 0, 17] = 2.0
+        qf[0, 1, 90] = -1.0
+    elif law == "constant_rows":       # every row equal: all scores tie, lowest ids win
+        kf[:] = kf[:, :, :1, :]
+    elif law == "sorted_scores":       # scores grow with the row id: the running threshold is
+        kf = np.abs(kf) * 0.01         # always stale and the best rows come last
+        qf = np.abs(qf)
+        kf *= np.linspace(0.5, 2.0, n, dtype=np.float32)[None, None, :, None]
+    elif law == "negative_scores":     # every score negative
+        kf = -np.abs(kf)
+        qf = np.abs(qf)
+    k, q = orc.f32_to_bf16(kf), orc.f32_to_bf16(qf)
+    for mode in (0, 1):
+        if law in ("huge",) and mode == 1:
+            continue                   # scores beyond 65536: outside the reference key's domain
+        check_sketch(k, q, 0, n, budget, mode, hip.ORDER_BEST)
+
+
 def test_sketch_select_ties_zero_query_and_group_mean():
     rng = np.random.default_rng(78)
     b, h, g, hd, n = 1, 3, 4, 128, 20000
