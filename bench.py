@@ -394,6 +394,27 @@ def main() -> int:
     def pct(p):
         return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
 
+    # Small configurations fit in the 256 MB Infinity Cache, so the loop above measures a
+    # warm cache.  Cold: a 1 GiB buffer is overwritten before every step (untimed) and each
+    # step is timed on its own.
+    cold_step_us = None
+    if n_units * L * region * hd * 2 < (512 << 20) and args.streams == 1:
+        flush = torch.empty((1 << 30,), dtype=torch.uint8, device=dev)
+        c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        cold = []
+        for s_i in range(min(args.steps, 30)):
+            with torch.cuda.stream(pipes[0].stream):
+                flush.fill_(s_i & 0xff)
+                c0.record()
+            step(events[s_i])
+            with torch.cuda.stream(pipes[0].stream):
+                c1.record()
+            torch.cuda.synchronize()
+            cold.append(c0.elapsed_time(c1) * 1e3)
+        cold.sort()
+        cold_step_us = cold[len(cold) // 2]
+        del flush
+
     graph_step_us = None
     if args.graph and args.streams == 1 and args.fused:
         # every call of the step only enqueues kernels on the stream, so the whole step can be
@@ -478,6 +499,7 @@ def main() -> int:
         "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
         "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
         "graph_step_us": graph_step_us,
+        "cold_cache_step_us_median": cold_step_us,
         "stage_us_per_layer": stage_us,
         "roofline": roofline,
         "setup_s": t_gen,
