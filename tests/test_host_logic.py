@@ -69,6 +69,33 @@ def test_invalid_arguments_are_reported_not_launched():
     assert rc == -12 and b"workspace" in _hip.lib.dc_last_error()
 
 
+def test_invalid_arguments_of_the_sketch_and_k_check_entry_points():
+    from diffcache_amd import _hip
+    lib = _hip.lib
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    # dc_sketch_build_bf16(k, codes, scale, resid, n_b, n_h, n_rows, hd, k strides, code strides, keep, stream)
+    rc = lib.dc_sketch_build_bf16(p, None, p, p, 1, 1, 4, 128, 0, 0, 128, 0, 0, 128, 0, None)
+    assert rc == -22 and b"null pointer" in lib.dc_last_error()
+    rc = lib.dc_sketch_build_bf16(p, p, p, p, 1, 1, 4, 96, 0, 0, 96, 0, 0, 96, 0, None)
+    assert rc == -22 and b"head_dim" in lib.dc_last_error()
+    rc = lib.dc_sketch_build_bf16(p, p, p, p, 1, 1, 4, 128, 0, 0, 128, 0, 0, 120, 0, None)
+    assert rc == -22 and b"code strides" in lib.dc_last_error()
+    # dc_score_select_sketch_bf16: bad order, then a workspace that is too small
+    args = [p, p, p, p, p, p, 8, 1, 1, 64, 128, 0, 0, 128, 0, 0, 128, 1, 8, 1]
+    rc = lib.dc_score_select_sketch_bf16(*args, 9, 0, p, 4096, None, None, None)
+    assert rc == -22 and b"order" in lib.dc_last_error()
+    rc = lib.dc_score_select_sketch_bf16(*args, 0, 0, p, 16, None, None, None)
+    assert rc == -12 and b"workspace" in lib.dc_last_error()
+    assert lib.dc_sketch_select_workspace_bytes(4, 1000, 16) == lib.dc_score_select_workspace_bytes(4, 1000, 16)
+    # dc_kcheck_f32: more sizes than the kernel takes, scores stride below n_sel
+    seq = (ctypes.c_int * 17)(*range(10, 27))
+    rc = lib.dc_kcheck_f32(p, 64, 1, 64, 128, 1, seq, 17, 0.9, p, None, None, None)
+    assert rc == -22 and b"at most 16" in lib.dc_last_error()
+    rc = lib.dc_kcheck_f32(p, 8, 1, 64, 128, 1, seq, 4, 0.9, p, None, None, None)
+    assert rc == -22 and b"scores_unit_stride" in lib.dc_last_error()
+
+
 def test_data_layer_option_errors():
     from diffcache_amd import DiffCacheHIP
     from diffcache_amd._hip import DiffCacheError
