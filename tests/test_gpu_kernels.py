@@ -443,6 +443,46 @@ def test_sketch_select_full_size_unit(mode):
     assert torch.equal(a, c)
 
 
+def test_select_routes_agree_on_random_cases():
+    """Dense scores + dc_topk_select, the streaming select and the sketch route must return
+    the same ids on randomly drawn shapes, budgets, key modes, orders and data laws."""
+    rng = np.random.default_rng(2024)
+    for it in range(400):
+        hd = int(rng.choice([64, 128, 256]))
+        b, h = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        grp = int(rng.choice([1, 1, 2, 4, 7]))
+        n = int(rng.choice([rng.integers(1, 600), rng.integers(600, 9000), rng.integers(9000, 70000)]))
+        budget = int(rng.choice([1, rng.integers(1, 64), rng.integers(64, 3000), rng.integers(3000, 9000)]))
+        lo, extra = int(rng.integers(0, 9)), int(rng.integers(0, 5))
+        mode, law = int(rng.integers(0, 2)), int(rng.integers(0, 6))
+        g = torch.Generator(device=DEV).manual_seed(int(rng.integers(1 << 30)))
+        k = torch.randn((b, h, lo + n + extra, hd), generator=g, device=DEV)
+        q = torch.randn((b, h * grp, hd), generator=g, device=DEV)
+        if law == 1:      # outlier channels
+            k = k * torch.exp(torch.randn((1, h, 1, hd), generator=g, device=DEV))
+        elif law == 2:    # many exact ties
+            k, q = torch.round(k * 2) / 2, torch.round(q)
+        elif law == 3:    # sparse keys
+            k = k * (torch.rand(k.shape, generator=g, device=DEV) < 0.1)
+        elif law == 4:    # scores grow with the row id
+            k = k.abs() * torch.linspace(0.2, 3.0, lo + n + extra, device=DEV)[None, None, :, None]
+            q = q.abs()
+        elif law == 5:    # one outlier row sets the sketch scales
+            k = k * 1e-3
+            k[:, :, lo + n // 2] = 50.0
+        k, q = k.to(torch.bfloat16).contiguous(), q.to(torch.bfloat16).contiguous()
+        order = int(rng.choice([hip.ORDER_BEST, hip.ORDER_INDEX]))
+        case = dict(it=it, hd=hd, b=b, h=h, grp=grp, n=n, budget=budget, lo=lo, mode=mode, law=law, order=order)
+        sk = hip.Sketch(k).build(k, lo, n)
+        dense = hip.score(k, q, lo, n, mode, q_group=grp)
+        a = hip.topk_select(dense, budget, mode, order)
+        s_ids = hip.score_select(k, q, lo, n, budget, mode, order, q_group=grp)
+        c = hip.score_select_sketch(k, sk, q, lo, n, budget, mode, order, q_group=grp)
+        ke = min(budget, n)
+        assert torch.equal(a[:, :ke], s_ids[:, :ke]), ("streaming", case)
+        assert torch.equal(a[:, :ke], c[:, :ke]), ("sketch", case)
+
+
 # ------------------------------------------------------------------ gather rows / kv maintenance
 
 def test_gather_rows_and_ingest_append():
