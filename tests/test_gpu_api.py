@@ -33,6 +33,24 @@ def bf16_close(got_f32, want_f64):
 
 # ---------------------------------------------------------------- DiffCacheHIP
 
+def test_data_layer_with_key_sketch_built_from_inserts_only():
+    """No prefill: the first insert fits the scales, later ones only raise the residual bounds."""
+    from diffcache_amd import DiffCacheHIP
+    rng = np.random.default_rng(34)
+    b, hkv, hd, n = 1, 2, 64, 40
+    dl = DiffCacheHIP(b, 2, hkv, hd, max_ctx_len=64, key_sketch=True)
+    ks = orc.f32_to_bf16(rng.integers(-9, 10, (n, b, hkv, hd)).astype(np.float32))
+    vs = rand_bf16(rng, n, b, hkv, hd)
+    for i in range(n):
+        dl.insert(ks[i], vs[i])
+    q = orc.f32_to_bf16(rng.integers(-2, 3, (b, hkv, hd)).astype(np.float32))
+    out_k = torch.zeros((b, hkv, 16, hd), dtype=torch.bfloat16, device=DEV)
+    out_v = torch.zeros_like(out_k)
+    dl.query(out_k, out_v, q, 16)
+    ck, cv, _ = cpu_ref.query(np.transpose(ks, (1, 2, 0, 3)).copy(), np.transpose(vs, (1, 2, 0, 3)).copy(), q, 16)
+    assert np.array_equal(np_u16(out_k), ck) and np.array_equal(np_u16(out_v), cv)
+
+
 def test_data_layer_with_key_sketch_follows_inserts():
     """key_sketch=True: same rows as the C restatement of the exact scan, also after rows far
     outside the range the sketch was fitted to have been inserted."""

@@ -629,6 +629,19 @@ def test_kcheck_matches_oracle(mode):
     kcheck_case(scores[:, :150], 64, [3, 5, 6, 100, 150, 200], 0.7, mode)   # sizes <= 5 and >= n_sel
 
 
+def test_kcheck_and_sketch_edge_sizes():
+    # no sizes to check -> the whole list; an empty list -> 0
+    sc = torch.sort(torch.randn((3, 40), device=DEV), dim=1, descending=True).values.contiguous()
+    assert hip.kcheck(sc, 40, 128, [], 0.9).tolist() == [40, 40, 40]
+    assert hip.kcheck(sc, 0, 128, [8, 16], 0.9).tolist() == [0, 0, 0]
+    # budget >= rows: every row is selected, in best-first order, through the sketch route too
+    rng = np.random.default_rng(12)
+    k, q = rand_bf16(rng, 1, 2, 300, 128), rand_bf16(rng, 1, 2, 128)
+    check_sketch(k, q, 0, 300, 300, 1, hip.ORDER_BEST)
+    check_sketch(k, q, 0, 300, 1000, 0, hip.ORDER_BEST)
+    check_sketch(k, q, 5, 1, 4, 1, hip.ORDER_BEST)
+
+
 def test_attention_identities_on_gpu():
     rng = np.random.default_rng(33)
     b, h, g, hd, n = 1, 2, 4, 128, 2500
