@@ -342,47 +342,59 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
     uint32_t wcnt = 0;
     const unsigned long long lt = (1ull << lane) - 1ull;
 
-    // Two steps (2 x 64 rows of this wave) are loaded together: a code row is half as
-    // long as a key row, so it takes twice the rows to keep as many bytes in flight.
-    for (int step = 0; step < steps; step += 2) {
+    // Double buffering: the loads of the next step are issued before the current step is
+    // worked on, so a wave always has a step's worth of bytes in flight.
+    auto load_step = [&](int step, uint4 (&cv)[LPR]) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
-        if (row0 >= n_rows) break;  // wave-uniform; no barrier inside the loop
-        const bool two = step + 1 < steps;
-        uint4 cv[2][LPR];
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-            if (s2 == 0 || two) {
-#pragma unroll
-                for (int j = 0; j < LPR; ++j) {
-                    int64_t r = row0 + (int64_t)s2 * kRowsPerBlockStep + grp * LPR + j;
-                    r = r > last ? last : r;
-                    cv[s2][j] = *reinterpret_cast<const uint4 *>(Cu + r * cr);
-                }
-            }
+        for (int j = 0; j < LPR; ++j) {
+            int64_t r = row0 + grp * LPR + j;
+            r = r > last ? last : r;
+            cv[j] = *reinterpret_cast<const uint4 *>(Cu + r * cr);
         }
-        uint32_t tb_next = tb;
-        if (step + 2 < steps) tb_next = load_relaxed(&st->tb_run);
+    };
+    auto work_step = [&](int step, const uint4 (&cv)[LPR]) {
+        const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
+        float mine = 0.f;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-            if (s2 == 0 || two) {
-                float mine = 0.f;
-#pragma unroll
-                for (int j = 0; j < LPR; ++j) {
-                    const float p = sketch_group_sum<LPR>(sketch_dot16(cv[s2][j], w, bias));
-                    mine = (col == j) ? p : mine;
-                }
-                const int64_t myrow = row0 + (int64_t)s2 * kRowsPerBlockStep + lane;
-                const bool valid = myrow < n_rows;
-                const uint32_t lb = dc_score_bucket(mine);
-                const bool keep = valid && dc_score_bucket(mine + margin) <= tb;
-                if (keep) atomicAdd(&lhist[lb], 1u);
-                const unsigned long long mask = __ballot(keep);
-                if (keep)
-                    wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
-                wcnt += (uint32_t)__popcll(mask);
-            }
+        for (int j = 0; j < LPR; ++j) {
+            const float p = sketch_group_sum<LPR>(sketch_dot16(cv[j], w, bias));
+            mine = (col == j) ? p : mine;
         }
+        const int64_t myrow = row0 + lane;
+        const bool valid = myrow < n_rows;
+        const uint32_t lb = dc_score_bucket(mine);
+        const bool keep = valid && dc_score_bucket(mine + margin) <= tb;
+        if (keep) atomicAdd(&lhist[lb], 1u);
+        const unsigned long long mask = __ballot(keep);
+        if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+        wcnt += (uint32_t)__popcll(mask);
+    };
+    // steps of this wave that hold rows (wave-uniform)
+    int my_steps = 0;
+    {
+        const int64_t first = block_row0 + wave * 64;
+        if (first < n_rows) {
+            const int64_t left = (int64_t)n_rows - first;
+            my_steps = (int)((left + kRowsPerBlockStep - 1) / kRowsPerBlockStep);
+            my_steps = my_steps < steps ? my_steps : steps;
+        }
+    }
+    uint4 ca[LPR], cb2[LPR];
+    if (my_steps > 0) load_step(0, ca);
+    // The threshold poll is issued before the prefetch: loads return in order, so waiting
+    // for a poll that was issued last would also wait for the whole prefetch.
+    for (int step = 0; step < my_steps; step += 2) {
+        uint32_t tb_next = load_relaxed(&st->tb_run);
+        if (step + 1 < my_steps) load_step(step + 1, cb2);
+        work_step(step, ca);
         tb = tb_next;
+        if (step + 1 < my_steps) {
+            tb_next = load_relaxed(&st->tb_run);
+            if (step + 2 < my_steps) load_step(step + 2, ca);
+            work_step(step + 1, cb2);
+            tb = tb_next;
+        }
     }
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
