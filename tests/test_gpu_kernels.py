@@ -443,6 +443,25 @@ def test_sketch_select_full_size_unit(mode):
     assert torch.equal(a, c)
 
 
+def test_select_routes_agree_on_1m_clustered_rows():
+    # the long-context benchmark shape: 2^20 rows in 256 tight clusters, k 4096, a query aimed at
+    # one cluster (its 4096 rows score almost alike: many candidates per unit)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    b, h, n, hd, k = 1, 2, 1 << 20, 128, 4096
+    centres = torch.randn((b, h, 256, hd), generator=g, device=DEV)
+    member = torch.randint(0, 256, (b, h, n), generator=g, device=DEV)
+    keys = torch.randn((b, h, n, hd), generator=g, device=DEV) * 0.1
+    for hi in range(h):
+        keys[0, hi] += centres[0, hi][member[0, hi]]
+    keys = keys.to(torch.bfloat16).contiguous()
+    q = (centres[:, :, 3] + 0.1 * torch.randn((b, h, hd), generator=g, device=DEV)).to(torch.bfloat16).contiguous()
+    sk = hip.Sketch(keys).build(keys, 4, n - 68)
+    for mode in (0, 1):
+        want = hip.topk_select(hip.score(keys, q, 4, n - 68, mode), k, mode, hip.ORDER_INDEX)
+        assert torch.equal(hip.score_select(keys, q, 4, n - 68, k, mode, hip.ORDER_INDEX), want)
+        assert torch.equal(hip.score_select_sketch(keys, sk, q, 4, n - 68, k, mode, hip.ORDER_INDEX), want)
+
+
 def test_select_routes_agree_on_random_cases():
     """Dense scores + dc_topk_select, the streaming select and the sketch route must return
     the same ids on randomly drawn shapes, budgets, key modes, orders and data laws."""
