@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the decode-time retrieval path on one MI355X.
 
-Workload (default): BASELINE.json configs[2] -- a full 32-layer Llama-3-8B-shaped
+Workload (default): benchmark configuration 3 -- a full 32-layer Llama-3-8B-shaped
 decode step, batch 8, context 131072 per sequence, 32 query / 8 kv heads,
 head_dim 128, bf16 K/V resident in HBM (~137 GB), top-k 2048 plus 4 sink tokens
 and a 64-token recent window.  One "step" = for every layer: score the whole
@@ -9,8 +9,15 @@ retrieval region with the GQA-mean query, select the exact top-k, run the
 gathered attention (including the current token's k/v).  Inputs are synthetic
 and already in HBM when the timed region starts.
 
-Prints ONE JSON line (see README / DESIGN for the fields).  `value` is the
-latency of one whole decode step in microseconds (lower is better).
+By default the scan reads the 8-bit sketch of the keys and rescans the rows that can
+still reach the top-k from the bf16 keys (same ids); --scan bf16 streams the bf16
+keys themselves.
+
+Prints ONE JSON line.  `value` is the latency of one whole decode step in
+microseconds (lower is better); `roofline` describes the scan kernel (bytes it must
+stream per launch over its measured duration, against the 8 TB/s HBM peak);
+`cpu_baseline` is the C restatement of the reference's exact scan timed on this
+machine's host cores.
 """
 from __future__ import annotations
 
@@ -139,7 +146,7 @@ def cpu_baseline(torch, cfg, layers_data, target_s: float = 10.0):
 
 
 def run_pq(args, torch, hip, dev) -> int:
-    """BASELINE config 4: PQ baseline, one layer, 8 kv heads x 1,048,576 keys, M 32 x 8-bit
+    """Benchmark configuration 4: PQ baseline, one layer, 8 kv heads x 1,048,576 keys, M 32 x 8-bit
     codes, ADC scan -> 4096 candidates -> exact bf16 rerank to top-k 1024."""
     from diffcache_amd.pq import PQIndex
     h, n, hd, m, n_cand, topk = 8, 1 << 20, 128, 32, 4096, 1024

@@ -745,7 +745,7 @@ def test_decode_layer_short_contexts():
 
 
 def test_decode_layer_config2_shape():
-    # BASELINE config 2: 32 q / 8 kv heads, hd 128, ctx 32768, k 1024, 4 sinks, 64 recent,
+    # benchmark configuration 2: 32 q / 8 kv heads, hd 128, ctx 32768, k 1024, 4 sinks, 64 recent,
     # keys with a per-channel log-normal scale
     rng = np.random.default_rng(2000)
     scale = np.exp(rng.standard_normal((1, 8, 1, 128))).astype(np.float32)

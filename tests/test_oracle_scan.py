@@ -189,7 +189,7 @@ def test_duplicate_rows_tie_to_lower_index():
 
 
 def test_planted_keys_fill_the_top(tmp_path):
-    # BASELINE config 1: N 8192, 16 planted keys = 3 q + 0.1 noise, k 256
+    # benchmark configuration 1: N 8192, 16 planted keys = 3 q + 0.1 noise, k 256
     rng = np.random.default_rng(1000)
     n, hd, k = 8192, 128, 256
     qf = rng.standard_normal(hd).astype(np.float32)
