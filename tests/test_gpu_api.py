@@ -491,3 +491,47 @@ def test_pq_index_search_matches_oracle_pipeline():
         assert np.array_equal(ids[u], cand[order])
         true = set(orc.topk_select(orc.scores_f32(q[u], keys[0, u]), 128, orc.MODE_IP).tolist())
         assert len(true & set(ids[u].tolist())) >= 40      # recall of ADC with 1024 candidates
+
+
+# ---------------------------------------------------------------- decode harness
+
+def test_harness_decode_step_matches_dense_attention():
+    """SyntheticLlama.decode_step around DiffCache.decode_attention: with a budget that covers
+    the whole retrieval region the sparse path is full attention, so the step must equal the
+    same layer stack computed with torch's own attention over the full key/value history."""
+    from diffcache_amd.harness import SyntheticLlama, synthetic_prompt_cache
+    from diffcache_amd import DiffCache
+    torch.manual_seed(0)
+    L, b, hq, hkv, hd, hidden, inter, ctx = 2, 2, 8, 2, 64, 256, 512, 300
+    model = SyntheticLlama(L, hidden, hq, hkv, hd, inter, device=DEV)
+    cache = DiffCache(num_layers=L, batch_size=b, max_length=ctx + 16, num_kv_heads=hkv, num_q_heads=hq,
+                      head_dim=hd, retrieval_budget=512, nsw_m=16, nsw_ef_cons=200, kvbuf_prefix_len=4,
+                      kvbuf_suffix_len=8, kvbuf_suffix_maxlen=24, attn_mass_threshold=0.9,
+                      k_check_seq=[1 << 30], r_sq=[[4.0] * hkv for _ in range(L)])
+    synthetic_prompt_cache(cache, ctx)
+    hist_k = [cache.kstore[l][:, :, :ctx].clone() for l in range(L)]       # (b, hkv, n, hd)
+    hist_v = [cache.vstore[l][:, :, :ctx].clone() for l in range(L)]
+    from diffcache_amd.harness import GraphedDecoder
+    x = torch.randn((b, hidden), device=DEV, dtype=torch.bfloat16)
+    g = hq // hkv
+    graphed = GraphedDecoder(model, cache, b)
+    for step in range(4):
+        pos = cache.seq_len(0)
+        assert pos == ctx + step
+        # eager on even steps, through the captured pre/post graphs on odd ones
+        got = (graphed.decode_step(x) if step % 2 else model.decode_step(cache, x)).clone()
+        # reference: the same stack with dense attention in fp32
+        xr = x
+        for l in range(L):
+            q, k, v = model.qkv(l, xr, pos)
+            hist_k[l] = torch.cat([hist_k[l], k.unsqueeze(2)], dim=2)
+            hist_v[l] = torch.cat([hist_v[l], v.unsqueeze(2)], dim=2)
+            kk = hist_k[l].float().repeat_interleave(g, dim=1)              # (b, hq, n, hd)
+            vv = hist_v[l].float().repeat_interleave(g, dim=1)
+            w = torch.softmax(torch.einsum("bhd,bhnd->bhn", q.float(), kk) / hd ** 0.5, dim=-1)
+            attn = torch.einsum("bhn,bhnd->bhd", w, vv).to(torch.bfloat16)
+            xr = model.post_attention(l, xr, attn)
+        err = (got.float() - xr.float()).abs().max().item()
+        scale = xr.float().abs().max().item()
+        assert err <= 0.03 * scale + 0.03, (step, err, scale)
+        x = got
