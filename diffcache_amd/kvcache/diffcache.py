@@ -24,6 +24,14 @@ own attention over ``get_kvcache()``.
 ``decode_attention`` is the native path that has no counterpart in the
 reference: score -> select -> attention straight from the store (one C call),
 replacing the ``flash_attn_with_kvcache`` call of ``base.py:134-142`` as well.
+
+Two options beyond the reference's arguments.  ``key_sketch`` (default on): an
+8-bit sketch of the keys is built at prefill and the scans read it instead of
+the bf16 keys, rescoring only the rows that can still reach the top-k; the ids
+are the same, the scan moves half the bytes (+25 % memory).  ``use_k_check``
+(default off): ``decode_attention`` applies the reference's k-check
+(``nsw.rs:198-296``, ``attn_mass_threshold``, ``k_check_seq``) to every unit's
+best-first result and attends only to the rows it finds sufficient.
 """
 from __future__ import annotations
 
