@@ -28,10 +28,11 @@ void dc_set_error(const char *fmt, ...);
         }                                                                  \
     } while (0)
 
-// select.hip: sort the selected ids of every unit (see the definition)
+// select.hip: sort the selected ids of every unit (see the definition); n_rows = rows of
+// the context the ids index into
 int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t *sel_keys,
                      uint32_t *idx_out, int64_t idx_stride, unsigned long long *scratch, int n_units,
-                     int k_eff, int mode, int order, hipStream_t st);
+                     int k_eff, int mode, int order, hipStream_t st, int n_rows);
 
 static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -873,7 +873,7 @@ int launch_finish(const char *who, const FusedWs &w, uint32_t *idx_out, int64_t 
     DC_CHECK_LAUNCH(who);
     if (order != DC_ORDER_ANY)
         return dc_sort_selected(nullptr, 0, sel_keys, idx_out, idx_unit_stride, w.sort_scratch, n_units,
-                                k_eff, mode, order, st);
+                                k_eff, mode, order, st, n_rows);
     return DC_OK;
 }
 

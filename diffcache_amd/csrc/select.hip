@@ -231,6 +231,48 @@ __global__ __launch_bounds__(kFinalThreads) void sort_kernel(
     for (int i = tid; i < k_eff; i += kFinalThreads) io[i] = (uint32_t)(buf[i] & 0xffffffffull);
 }
 
+// DC_ORDER_INDEX without a sort: the unit's ids are marked in an LDS bitmap of the
+// context (one bit per row) and read back in ascending order.  One block per unit;
+// used while the bitmap fits in LDS (2^20 rows = 128 KB).
+constexpr int kBitmapMaxRows = 1 << 20;
+
+__global__ __launch_bounds__(kFinalThreads) void index_order_kernel(uint32_t *__restrict__ idx_out,
+                                                                    int64_t idx_stride, int k_eff,
+                                                                    int n_words) {
+    extern __shared__ uint32_t bitmap[];
+    __shared__ uint32_t wtot[kFinalThreads / 64 + 1];
+    const int unit = blockIdx.x;
+    const int tid = threadIdx.x;
+    uint32_t *io = idx_out + (int64_t)unit * idx_stride;
+    // word w lives at w + w/32: the runs of 32 words the threads sweep below then start in
+    // different banks
+    auto slot = [](int w) { return w + (w >> 5); };
+    const int n_slots = slot(n_words - 1) + 1;
+    for (int i = tid; i < n_slots; i += kFinalThreads) bitmap[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < k_eff; i += kFinalThreads) {
+        const uint32_t id = io[i];
+        atomicOr(&bitmap[slot((int)(id >> 5))], 1u << (id & 31u));
+    }
+    __syncthreads();
+    // every thread owns a contiguous run of words
+    const int per = (n_words + kFinalThreads - 1) / kFinalThreads;
+    const int w0 = tid * per;
+    const int w1 = w0 + per < n_words ? w0 + per : n_words;
+    uint32_t cnt = 0;
+    for (int w = w0; w < w1; ++w) cnt += __popc(bitmap[slot(w)]);
+    uint32_t total;
+    uint32_t pos = block_excl_scan<kFinalThreads>(cnt, wtot, &total);
+    for (int w = w0; w < w1; ++w) {
+        uint32_t bits = bitmap[slot(w)];
+        while (bits) {
+            const int b = __ffs((int)bits) - 1;
+            io[pos++] = (uint32_t)w * 32u + (uint32_t)b;
+            bits &= bits - 1u;
+        }
+    }
+}
+
 __global__ void compose_idx_kernel(const uint32_t *__restrict__ outer, int64_t outer_stride,
                                    const uint32_t *__restrict__ inner, int64_t inner_stride,
                                    uint32_t *__restrict__ out, int64_t out_stride, int n_inner,
@@ -281,7 +323,23 @@ SelectWs carve(void *base, int n_units, int n_rows, int k) {
 // scores; DC_ORDER_INDEX by id.  scratch is needed when k_eff > 4096.
 int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t *sel_keys,
                      uint32_t *idx_out, int64_t idx_stride, unsigned long long *scratch, int n_units,
-                     int k_eff, int mode, int order, hipStream_t st) {
+                     int k_eff, int mode, int order, hipStream_t st, int n_rows) {
+    if (order == DC_ORDER_INDEX && n_rows > 0 && n_rows <= kBitmapMaxRows && k_eff >= 512) {
+        // the ids are distinct and below n_rows: mark and sweep beats a bitonic sort
+        const int n_words = (n_rows + 31) / 32;
+        const size_t lds = (size_t)(n_words + (n_words >> 5) + 1) * 4;
+        static bool attr_set = false;
+        if (!attr_set) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(index_order_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (kBitmapMaxRows / 32 + kBitmapMaxRows / 1024 + 1) * 4);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(index_order_kernel, dim3(n_units), dim3(kFinalThreads), lds, st, idx_out,
+                           idx_stride, k_eff, n_words);
+        DC_CHECK_LAUNCH("dc_sort_selected(index)");
+        return DC_OK;
+    }
     const int p2 = next_pow2(k_eff);
     if (p2 <= kSortLds)
         hipLaunchKernelGGL(sort_kernel<true>, dim3(n_units), dim3(kFinalThreads), 0, st, scores,
@@ -345,7 +403,7 @@ extern "C" int dc_topk_select(const float *scores, int64_t scores_unit_stride, u
     DC_CHECK_LAUNCH("dc_topk_select(finalize)");
     if (order != DC_ORDER_ANY)
         return dc_sort_selected(scores, scores_unit_stride, nullptr, idx_out, idx_unit_stride,
-                                w.sort_scratch, n_units, k_eff, mode, order, st);
+                                w.sort_scratch, n_units, k_eff, mode, order, st, n_rows);
     return DC_OK;
 }
 
