@@ -160,20 +160,33 @@ def run_pq(args, torch, hip, dev) -> int:
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps)]
 
     def step(e=None):
+        if args.stepwise:
+            return step_stepwise(e)
         lut = hip.pq_build_lut(q, index.books, 1)
-        index.hist.zero_()
+        ids = hip.pq_search(store, index.codes, lut, q, n_cand, topk, idx_out=index.ids,
+                            workspace=index.ws, state_ready=index._ws_ready, scan_events=e)
+        index._ws_ready = True
+        return ids
+
+    hist = hip.new_hist(h, dev)
+
+    def step_stepwise(e=None):
+        # the separate entry points, with a dense ADC score array
+        lut = hip.pq_build_lut(q, index.books, 1)
+        hist.zero_()
         if e is not None:
             e[0].record()
-        adc = hip.pq_adc_scan(index.codes, lut, hist=index.hist)
+        adc = hip.pq_adc_scan(index.codes, lut, hist=hist)
         if e is not None:
             e[1].record()
-        cand = hip.topk_select(adc, n_cand, hip.MODE_IP, hip.ORDER_INDEX, hist=index.hist,
-                               idx_out=index.cand, workspace=index.ws1)
+        cand = hip.topk_select(adc, n_cand, hip.MODE_IP, hip.ORDER_INDEX, hist=hist)
         exact = hip.score_gathered(store, q, cand)
-        pos = hip.topk_select(exact, topk, hip.MODE_IP, hip.ORDER_BEST, idx_out=index.pos,
-                              workspace=index.ws2)
+        pos = hip.topk_select(exact, topk, hip.MODE_IP, hip.ORDER_BEST)
         return hip.compose_idx(cand, pos)
 
+    for e in ev:            # events must exist before the library records them
+        e[0].record()
+        e[1].record()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -193,7 +206,8 @@ def run_pq(args, torch, hip, dev) -> int:
         "config": {"workload": "config4: PQ baseline, 8 kv heads x 1048576 keys, hd 128, M 32 x 256 centroids, "
                                "ADC scan -> 4096 candidates -> exact rerank to top-k 1024"},
         "roofline": {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": ach / HBM_PEAK_GBPS, "traffic": None, "kernel": "pq_adc_kernel<32>",
+                     "frac": ach / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "pq_adc_kernel<32>" if args.stepwise else "pq_prune_kernel<32>",
                      "algorithmic_bytes_per_launch": scan_bytes, "avg_launch_us": scan_ms * 1e3},
         "cpu_baseline": None, "setup_s": t_gen}))
     return 0
@@ -222,6 +236,9 @@ def main() -> int:
     ap.add_argument("--dense", action="store_true",
                     help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
                          "streaming score + select")
+    ap.add_argument("--stepwise", action="store_true",
+                    help="config c4 only: the PQ search through the separate entry points (dense ADC "
+                         "score array) instead of dc_pq_search_bf16")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one decode step (all layers) in a HIP graph and time its replays; "
                          "reported as graph_step_us next to the eager figure")

@@ -34,6 +34,7 @@ SYMBOLS = (
     "dc_sparse_select", "dc_score_select_bf16",
     "dc_sketch_build_bf16", "dc_sketch_select_workspace_bytes", "dc_sketch_select_state_init",
     "dc_score_select_sketch_bf16", "dc_kcheck_f32",
+    "dc_pq_search_workspace_bytes", "dc_pq_search_bf16",
 )
 
 
@@ -84,6 +85,8 @@ def _load() -> C.CDLL:
         "dc_pq_adc_scan": (i, [p, p, p, p, i, i, i, i64, p]),
         "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
         "dc_compose_idx": (i, [p, i64, p, i64, p, i64, i, i, p]),
+        "dc_pq_search_workspace_bytes": (sz, [i, i, i]),
+        "dc_pq_search_bf16": (i, [p, p, p, p, p, i64, i, i, i, i, i, i64, i64, i64, i, i, i, p, sz, p, p, p]),
         "dc_score_select_workspace_bytes": (sz, [i, i, i]),
         "dc_select_state_init": (i, [i, i, i, p, sz, p]),
         "dc_score_prune_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i, i, i, p, sz, p]),
@@ -494,6 +497,34 @@ def pq_adc_scan(codes: torch.Tensor, lut: torch.Tensor, hist: Optional[torch.Ten
     _check(lib.dc_pq_adc_scan(_dev(codes, "codes"), _dev(lut, "lut"), _dev(scores, "scores"),
                               _opt(hist, "hist"), n_units, n_rows, m, scores.stride(0), _stream()))
     return scores
+
+
+def pq_search(store_k: torch.Tensor, codes: torch.Tensor, lut: torch.Tensor, q: torch.Tensor,
+              n_cand: int, topk: int, idx_out: Optional[torch.Tensor] = None,
+              workspace: Optional[torch.Tensor] = None, state_ready: bool = False,
+              scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None) -> torch.Tensor:
+    """ADC scan -> n_cand candidates -> exact rerank -> topk ids, best first, in one call
+    (dc_pq_search_bf16).  store_k (b, h, n, hd) bf16, codes (b*h, n, M) uint8,
+    lut (b*h, M, 256) fp32, q (b*h, hd) bf16 -> int32 (b*h, min(topk, n))."""
+    sb, sh, sr = _store_strides(store_k)
+    b, h, n, hd = store_k.shape
+    n_units, n_rows, m = codes.shape
+    if n_units != b * h or n_rows != n:
+        raise ValueError("codes do not match the key store")
+    codes, lut, q = codes.contiguous(), lut.contiguous(), q.contiguous()
+    k2 = min(topk, n_cand, n)
+    if idx_out is None:
+        idx_out = torch.empty((n_units, k2), dtype=torch.int32, device=q.device)
+    need = lib.dc_pq_search_workspace_bytes(n_units, n, n_cand)
+    if workspace is None:
+        workspace = alloc_workspace(need, q.device)
+    _check(lib.dc_pq_search_bf16(_dev(store_k, "store_k"), _dev(codes, "codes"), _dev(lut, "lut"),
+                                 _dev(q, "q"), _dev(idx_out, "idx_out"), idx_out.stride(0), b, h, n, hd, m,
+                                 sb, sh, sr, n_cand, topk, int(state_ready), _dev(workspace, "workspace"),
+                                 workspace.numel() * workspace.element_size(),
+                                 scan_events[0].cuda_event if scan_events else None,
+                                 scan_events[1].cuda_event if scan_events else None, _stream()))
+    return idx_out
 
 
 def score_gathered(store_k: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, row_offset: int = 0,

@@ -30,6 +30,7 @@
 // select_finish_kernel picks the k best of that list.
 #include "dc_common.h"
 #include "dc_select.h"
+#include "dc_pq.h"
 
 namespace {
 
@@ -39,6 +40,8 @@ constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
+constexpr int kPqThreads = 512;    // PQ scan: threads per block = keys per step
+constexpr int kPqBigSteps = 8;     // PQ scan: 4096 keys per large block
 constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
 static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kThreads == DC_HIST_BINS, "bin split");
 
@@ -76,10 +79,21 @@ __device__ __forceinline__ uint32_t load_relaxed(const uint32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// A block's copy of its unit's running threshold bucket, in LDS.  The poll of the unit's
+// value crosses the chip (agent scope) and every younger load of the polling wave returns
+// after it, so one wave of the block polls and the others read the copy.
+__device__ __forceinline__ uint32_t lds_load_relaxed(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_store_relaxed(uint32_t *p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // End of a scan block: append the block's survivors (staged per wave in LDS) to
 // the unit's list with one returning atomic, flush the block's histogram, and in
 // the blocks chosen by the caller refresh the unit's running threshold from
 // whatever part of the histogram is visible.  Staleness only loosens the bound.
+template <int kT = kThreads>
 __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 *wstage, uint32_t wcnt,
                                                    uint32_t *s_wcnt, uint32_t *s_base, uint32_t *wtot,
                                                    UnitState *st, uint32_t *hu, uint2 *surv_unit,
@@ -92,12 +106,12 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
     // the atomic is in flight while the histogram is flushed
     uint32_t wbase = 0, cnt = 0;
 #pragma unroll
-    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+    for (int w2 = 0; w2 < kT / 64; ++w2) {
         if (w2 < wave) wbase += s_wcnt[w2];
         cnt += s_wcnt[w2];
     }
     if (tid == 0) *s_base = cnt ? atomicAdd(&st->surv_cnt, cnt) : 0;
-    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
+    for (int i = tid; i < DC_HIST_BINS; i += kT) {
         const uint32_t c = lhist[i];
         if (c) atomicAdd(&hu[i], c);
     }
@@ -113,26 +127,28 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
     {
         const unsigned long long *h64 = reinterpret_cast<const unsigned long long *>(hu);
         unsigned long long *l64 = reinterpret_cast<unsigned long long *>(lhist);
-        for (int i = tid; i < DC_HIST_BINS / 2; i += kThreads)
+        for (int i = tid; i < DC_HIST_BINS / 2; i += kT)
             l64[i] = __hip_atomic_load(h64 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    uint32_t bins[kBinsPerThread];
+    constexpr int kBins = DC_HIST_BINS / kT;  // adjacent bins a thread owns
+    static_assert(kBins * kT == DC_HIST_BINS, "bin split");
+    uint32_t bins[kBins];
     uint32_t sum = 0;
 #pragma unroll
-    for (int i = 0; i < kBinsPerThread; ++i) {
-        bins[i] = lhist[tid * kBinsPerThread + i];
+    for (int i = 0; i < kBins; ++i) {
+        bins[i] = lhist[tid * kBins + i];
         sum += bins[i];
     }
     uint32_t total;
-    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
+    const uint32_t excl = block_excl_scan<kT>(sum, wtot, &total);
     if (excl < kk && kk <= excl + sum) {
         uint32_t run = excl;
         bool done = false;
 #pragma unroll
-        for (int i = 0; i < kBinsPerThread; ++i) {
+        for (int i = 0; i < kBins; ++i) {
             if (!done && run + bins[i] >= kk) {
-                atomicMin(&st->tb_run, (uint32_t)(tid * kBinsPerThread + i));
+                atomicMin(&st->tb_run, (uint32_t)(tid * kBins + i));
                 done = true;
             }
             run += bins[i];
@@ -401,6 +417,117 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
                        surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
 }
 
+// The same scan for the PQ baseline: a key's score is its ADC score (dc_pq.h), read
+// from M code bytes per key, in DC_MODE_IP order.  One key per lane.  The unit's
+// tables are staged per block, so blocks are large: 512 threads, 512 keys per step.
+template <int M>
+__global__ __launch_bounds__(kPqThreads) void pq_prune_kernel(
+    const uint8_t *__restrict__ codes, const float *__restrict__ lut, uint32_t *__restrict__ hist,
+    UnitState *__restrict__ state, uint2 *__restrict__ surv, int n_units, int n_rows, int k_eff,
+    int small_chunks, int big_steps) {
+    constexpr int NW = M / 4;
+    constexpr int kWaves = kPqThreads / 64;
+    __shared__ float s_lut[kPqLutWords];
+    __shared__ uint32_t lhist[DC_HIST_BINS];
+    __shared__ uint2 stage[kWaves * kPqBigSteps * 64];
+    __shared__ uint32_t s_tb;  // the block's copy of the unit's running threshold bucket
+    __shared__ uint32_t wtot[kWaves + 1];
+    __shared__ uint32_t s_wcnt[kWaves];
+    __shared__ uint32_t s_base;
+
+    const int unit = blockIdx.x % n_units;
+    const int chunk = blockIdx.x / n_units;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const bool small = chunk < small_chunks;
+    const int big_chunks = (int)(gridDim.x / n_units) - small_chunks;
+    const int big_id = small ? 0 : (int)(((int64_t)(chunk - small_chunks) + (int64_t)unit * 7) % big_chunks);
+    const int64_t block_row0 =
+        small ? (int64_t)chunk * kPqThreads
+              : (int64_t)small_chunks * kPqThreads + (int64_t)big_id * big_steps * kPqThreads;
+    const int steps = small ? 1 : big_steps;
+
+    for (int i = tid; i < DC_HIST_BINS; i += kPqThreads) lhist[i] = 0;
+    pq_stage_lut<M>(s_lut, lut + (int64_t)unit * M * 256, tid, kPqThreads);
+    PqLane<M> ln;
+    ln.init(lane);
+    UnitState *st = state + unit;
+    const int64_t last = n_rows - 1;
+    uint32_t tb = load_relaxed(&st->tb_run);
+    const uint8_t *cu = codes + (int64_t)unit * n_rows * M;
+    // rows are a multiple of 64 from the start of the unit: lane = key mod 64, as pq_adc_score expects
+    const int64_t blk_end = block_row0 + (int64_t)steps * kPqThreads - 1;
+    const int64_t blk_last = blk_end < last ? blk_end : last;
+    auto load_row = [&](int64_t row0, uint32_t(&w)[NW]) {
+        int64_t r = row0 + lane;
+        r = r > blk_last ? blk_last : r;
+        const uint4 *cp = reinterpret_cast<const uint4 *>(cu + r * M);
+#pragma unroll
+        for (int i = 0; i < NW / 4; ++i) {
+            const uint4 t = cp[i];
+            w[4 * i + 0] = t.x;
+            w[4 * i + 1] = t.y;
+            w[4 * i + 2] = t.z;
+            w[4 * i + 3] = t.w;
+        }
+    };
+    // A wave keeps the codes of kAhead steps in flight beyond the one it scores: 32 bytes
+    // per lane and step are too few to cover the memory latency otherwise.  Loads return
+    // in order, so the threshold polled before the rows of step s + kAhead is first looked
+    // at when those rows are, and never makes the wave wait for younger loads.  The
+    // requests are issued unconditionally (past the block's end they repeat its last
+    // row) so that the number of loads in flight is the same on every path.
+    constexpr int kAhead = 3, kRing = kAhead + 1;
+    uint32_t buf[kRing][NW];
+    const int64_t wave_row0 = block_row0 + wave * 64;
+    const int64_t rows_left = (int64_t)n_rows - wave_row0;
+    const int64_t steps_left = (rows_left + kPqThreads - 1) / kPqThreads;
+    const int my_steps = rows_left <= 0 ? 0 : (int)(steps_left < steps ? steps_left : steps);
+    uint32_t tb_polled = tb;
+    if (tid == 0) s_tb = tb;
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) load_row(wave_row0 + (int64_t)j * kPqThreads, buf[j]);
+    __syncthreads();
+
+    // each wave stages its survivors in its own slice (at most 64 per step)
+    uint2 *wstage = stage + wave * (kPqBigSteps * 64);
+    uint32_t wcnt = 0;
+    const unsigned long long lt = (1ull << lane) - 1ull;
+
+    for (int s0 = 0; s0 < my_steps; s0 += kRing) {
+#pragma unroll
+        for (int j = 0; j < kRing; ++j) {
+            const int step = s0 + j;
+            const int64_t row0 = wave_row0 + (int64_t)step * kPqThreads;
+            // The poll crosses the chip (agent scope) and every younger load of the wave
+            // queues behind it, so only wave 0 polls, once per kRing steps, and hands the
+            // value to the other waves through LDS when it has arrived.
+            if (wave == 0 && j == 0) tb_polled = load_relaxed(&st->tb_run);
+            load_row(row0 + (int64_t)kAhead * kPqThreads, buf[(j + kAhead) % kRing]);
+            if (wave == 0 && j == kAhead && lane == 0) lds_store_relaxed(&s_tb, tb_polled);
+            if (step < my_steps) {  // wave-uniform; no barrier inside the loop
+                const float mine = pq_adc_score<M>(buf[j], s_lut, ln);
+                tb = lds_load_relaxed(&s_tb);
+                const int64_t myrow = row0 + lane;
+                const bool valid = myrow < n_rows;
+                uint32_t key = 0, bucket = 0xffffffffu;
+                if (valid) dc_key_bucket(mine, DC_MODE_IP, key, bucket);
+                const bool keep = valid && bucket <= tb;
+                if (keep) atomicAdd(&lhist[bucket], 1u);
+                const unsigned long long mask = __ballot(keep);
+                if (keep)
+                    wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+                wcnt += (uint32_t)__popcll(mask);
+            }
+        }
+    }
+    // every 4th small block and every 2nd large one refresh the running threshold
+    const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 1) == 1;
+    prune_block_finish<kPqThreads>(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st,
+                                   hist + (int64_t)unit * DC_HIST_BINS, surv + (int64_t)unit * n_rows,
+                                   refresh, (uint32_t)k_eff);
+}
+
 // Exact threshold bucket of a unit from its complete histogram: the bucket that
 // holds the k-th best key, and how many keys sit in better buckets.  Called by
 // all kThreads threads; the result is uniform.  `wtot`, `sres`: LDS scratch.
@@ -641,6 +768,41 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     }
 }
 
+// Exact scores of the rows the PQ scan selected: one LPR-lane group per row, the
+// arithmetic of score_gathered_kernel.  Their (key, id) become the unit's candidate
+// list, from which select_finish_kernel picks the best (c_less = 0).
+template <int HD>
+__global__ __launch_bounds__(kThreads) void pq_rescore_kernel(
+    const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, const uint32_t *__restrict__ idx,
+    UnitState *__restrict__ state, uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_idx,
+    int n_h, int n_idx, int64_t idx_stride, int n_rows, int64_t sb, int64_t sh, int64_t sr,
+    int blocks_per_unit) {
+    constexpr int LPR = HD / 8;
+    constexpr int GROUPS = kThreads / LPR;
+    const int unit = blockIdx.x / blocks_per_unit;
+    const int chunk = blockIdx.x % blocks_per_unit;
+    const int b = unit / n_h, h = unit % n_h;
+    const int grp = threadIdx.x / LPR, col = threadIdx.x % LPR;
+    if (chunk == 0 && threadIdx.x == 0) {
+        state[unit].cand_cnt = (uint32_t)n_idx;
+        state[unit].c_less = 0;
+    }
+    float q[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = dc_bf16_to_f32(Q[(int64_t)unit * HD + col * 8 + i]);
+    const int j = chunk * GROUPS + grp;
+    const int jj = j < n_idx ? j : n_idx - 1;
+    const uint32_t id = idx[(int64_t)unit * idx_stride + jj];
+    const uint4 w = *reinterpret_cast<const uint4 *>(K + b * sb + h * sh + (int64_t)id * sr + col * 8);
+    const float p = dc_group_sum<LPR>(dc_dot8(w, q, 0.f));
+    if (j < n_idx && col == 0) {
+        uint32_t key, bucket;
+        dc_key_bucket(p, DC_MODE_IP, key, bucket);
+        cand_key[(int64_t)unit * n_rows + j] = key;
+        cand_idx[(int64_t)unit * n_rows + j] = id;
+    }
+}
+
 // One block per unit: radix select among the candidates of the threshold bucket
 // fills idx_out[c_less, k).  Leaves the unit's list cursors at zero.
 __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
@@ -785,18 +947,19 @@ struct FusedPlan {
     int64_t blocks;
 };
 
-int plan_fused(const char *who, int n_b, int n_h, int n_rows, int budget, FusedPlan *p) {
+int plan_fused(const char *who, int n_b, int n_h, int n_rows, int budget, FusedPlan *p,
+               int big_steps = kBigSteps, int rows_per_step = kRowsPerBlockStep) {
     DC_REQUIRE(n_b >= 0 && n_h >= 1 && n_rows >= 0 && budget >= 0, "%s: bad sizes", who);
     const int64_t n_units64 = (int64_t)n_b * n_h;
     DC_REQUIRE(n_units64 < (1 << 20), "%s: too many units", who);
     p->n_units = (int)n_units64;
     p->k_eff = budget < n_rows ? budget : n_rows;
-    // chunks per unit: up to kSmallChunks blocks of 256 rows, then blocks of 2048 rows
-    const int64_t tiles = ((int64_t)n_rows + kRowsPerBlockStep - 1) / kRowsPerBlockStep;
-    p->big_steps = kBigSteps;
+    // chunks per unit: up to kSmallChunks blocks of one step, then blocks of big_steps steps
+    const int64_t tiles = ((int64_t)n_rows + rows_per_step - 1) / rows_per_step;
+    p->big_steps = big_steps;
     p->small_chunks = (int)(tiles < kSmallChunks ? tiles : kSmallChunks);
-    const int64_t rest = (int64_t)n_rows - (int64_t)p->small_chunks * kRowsPerBlockStep;
-    const int64_t big_rows = (int64_t)p->big_steps * kRowsPerBlockStep;
+    const int64_t rest = (int64_t)n_rows - (int64_t)p->small_chunks * rows_per_step;
+    const int64_t big_rows = (int64_t)p->big_steps * rows_per_step;
     const int64_t big_chunks = rest > 0 ? (rest + big_rows - 1) / big_rows : 0;
     p->blocks = n_units64 * (p->small_chunks + big_chunks);
     DC_REQUIRE(p->blocks < (1ll << 31), "%s: grid too large", who);
@@ -996,4 +1159,74 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
 #undef DC_LAUNCH_RS
     DC_CHECK_LAUNCH(who);
     return launch_finish(who, w, idx_out, idx_unit_stride, p.n_units, n_rows, p.k_eff, mode, order, 1, st);
+}
+
+extern "C" size_t dc_pq_search_workspace_bytes(int n_units, int n_rows, int n_cand) {
+    const FusedWs w = carve_fused(nullptr, n_units, n_rows, n_cand);
+    const size_t nu = n_units > 0 ? n_units : 0;
+    const size_t kc = (size_t)(n_cand < n_rows ? n_cand : n_rows);
+    return w.bytes + dc_align_up(nu * (n_cand > 0 && n_rows > 0 ? kc : 0) * 4, 256);
+}
+
+extern "C" int dc_pq_search_bf16(const void *k, const uint8_t *codes, const float *lut, const void *q,
+                                 uint32_t *idx_out, int64_t idx_unit_stride, int n_b, int n_h, int n_rows,
+                                 int hd, int m, int64_t sb, int64_t sh, int64_t sr, int n_cand, int topk,
+                                 int state_ready, void *workspace, size_t workspace_bytes,
+                                 void *ev_scan_begin, void *ev_scan_end, void *stream) {
+    const char *who = "dc_pq_search_bf16";
+    DC_REQUIRE(k && codes && lut && q && idx_out, "%s: null pointer", who);
+    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d not in {64,128,256}", who, hd);
+    DC_REQUIRE(m == 16 || m == 32, "%s: m = %d subspaces unsupported (16 or 32)", who, m);
+    DC_REQUIRE(n_cand >= 0 && topk >= 0 && topk <= n_cand, "%s: need 0 <= topk <= n_cand", who);
+    DC_REQUIRE(dc_aligned16(k) && dc_aligned16(codes) && dc_aligned16(lut),
+               "%s: k, codes and lut must be 16-byte aligned", who);
+    DC_REQUIRE(sb % 8 == 0 && sh % 8 == 0 && sr % 8 == 0 && sr >= hd,
+               "%s: key strides must be multiples of 8 elements and row_stride >= hd", who);
+    FusedPlan p;
+    int rc = plan_fused(who, n_b, n_h, n_rows, n_cand, &p, kPqBigSteps, kPqThreads);
+    if (rc) return rc;
+    const int k1 = p.k_eff;                   // candidates per unit
+    const int k2 = topk < k1 ? topk : k1;     // results per unit
+    if (p.n_units == 0 || k2 == 0) return DC_OK;
+    DC_REQUIRE(idx_unit_stride >= k2, "%s: idx_unit_stride < min(topk, n_rows)", who);
+    DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
+               "%s: workspace must be non-null and 256-byte aligned", who);
+    const FusedWs w = carve_fused(workspace, p.n_units, n_rows, n_cand);
+    const size_t need = dc_pq_search_workspace_bytes(p.n_units, n_rows, n_cand);
+    if (workspace_bytes < need) {
+        dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, need);
+        return DC_ENOMEM;
+    }
+    uint32_t *cand = (uint32_t *)((char *)workspace + w.bytes);
+    hipStream_t st = (hipStream_t)stream;
+    if (!state_ready) {
+        rc = dc_select_state_init(p.n_units, n_rows, n_cand, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+    }
+    if (ev_scan_begin) (void)hipEventRecord((hipEvent_t)ev_scan_begin, st);
+    if (m == 16)
+        hipLaunchKernelGGL(pq_prune_kernel<16>, dim3((unsigned)p.blocks), dim3(kPqThreads), 0, st, codes, lut,
+                           w.hist, w.state, w.surv, p.n_units, n_rows, k1, p.small_chunks, p.big_steps);
+    else
+        hipLaunchKernelGGL(pq_prune_kernel<32>, dim3((unsigned)p.blocks), dim3(kPqThreads), 0, st, codes, lut,
+                           w.hist, w.state, w.surv, p.n_units, n_rows, k1, p.small_chunks, p.big_steps);
+    DC_CHECK_LAUNCH(who);
+    if (ev_scan_end) (void)hipEventRecord((hipEvent_t)ev_scan_end, st);
+    // the k1 best ADC scores of every unit, in no particular order
+    rc = launch_select(who, w, cand, k1, p.n_units, n_rows, k1, DC_MODE_IP, DC_ORDER_ANY, 1, st);
+    if (rc) return rc;
+    const int lpr = hd / 8, groups = kThreads / lpr;
+    const int64_t bpu = ((int64_t)k1 + groups - 1) / groups;
+    DC_REQUIRE((int64_t)p.n_units * bpu < (1ll << 31), "%s: grid too large", who);
+#define DC_LAUNCH_PR(HD)                                                                              \
+    hipLaunchKernelGGL(pq_rescore_kernel<HD>, dim3((unsigned)(p.n_units * bpu)), dim3(kThreads), 0, st, \
+                       (const uint16_t *)k, (const uint16_t *)q, cand, w.state, w.cand_key, w.cand_idx, \
+                       n_h, k1, (int64_t)k1, n_rows, sb, sh, sr, (int)bpu)
+    if (hd == 64) DC_LAUNCH_PR(64);
+    else if (hd == 128) DC_LAUNCH_PR(128);
+    else DC_LAUNCH_PR(256);
+#undef DC_LAUNCH_PR
+    DC_CHECK_LAUNCH(who);
+    return launch_finish(who, w, idx_out, idx_unit_stride, p.n_units, n_rows, k2, DC_MODE_IP, DC_ORDER_BEST, 1,
+                         st);
 }

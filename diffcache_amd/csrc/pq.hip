@@ -3,11 +3,11 @@
 // (evaluation/impl/pqcache) is empty, so this follows the benchmark
 // configuration only: M subspaces x 256 centroids, 8-bit codes, fp32 tables.
 //
-// The scan keeps the unit's whole table (M * 256 floats, 32 KB at M 32) in LDS
-// and gives each thread one key at a time: M code bytes, M table reads, M fp32
-// adds in ascending subspace order.  HBM traffic is M bytes per key; the LDS
-// gathers (4*M bytes per key, random banks) are what bounds it in practice.
+// The scan keeps the unit's tables in LDS (32 KB, laid out so that the reads of a
+// wave never share a bank, see dc_pq.h) and gives each thread one key at a time:
+// M code bytes, M table reads, M fp32 adds.  HBM traffic is M bytes per key.
 #include "dc_common.h"
+#include "dc_pq.h"
 
 namespace {
 
@@ -34,39 +34,34 @@ template <int M>
 __global__ __launch_bounds__(kThreads) void pq_adc_kernel(
     const uint8_t *__restrict__ codes, const float *__restrict__ lut, float *__restrict__ scores,
     uint32_t *__restrict__ hist, int n_rows, int64_t scores_stride, int blocks_per_unit) {
-    __shared__ float s_lut[M * 256];
+    __shared__ float s_lut[kPqLutWords];
     __shared__ uint32_t lhist[DC_HIST_BINS];
     const int unit = blockIdx.x / blocks_per_unit;
     const int chunk = blockIdx.x % blocks_per_unit;
     const int tid = threadIdx.x;
-    {
-        const float4 *src = reinterpret_cast<const float4 *>(lut + (int64_t)unit * M * 256);
-        float4 *dst = reinterpret_cast<float4 *>(s_lut);
-        for (int i = tid; i < M * 64; i += kThreads) dst[i] = src[i];
-    }
+    pq_stage_lut<M>(s_lut, lut + (int64_t)unit * M * 256, tid, kThreads);
     if (hist)
         for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
+    PqLane<M> ln;
+    ln.init(tid & 63);
     __syncthreads();
     const uint8_t *cu = codes + (int64_t)unit * n_rows * M;
     float *su = scores + (int64_t)unit * scores_stride;
-    const int64_t base = (int64_t)chunk * kKeysPerBlock;
+    const int64_t base = (int64_t)chunk * kKeysPerBlock;  // a multiple of 64: lane = key mod 64
     for (int it = 0; it < kKeysPerThread; ++it) {
         const int64_t i = base + (int64_t)it * kThreads + tid;
         if (i >= n_rows) break;
         const uint4 *cp = reinterpret_cast<const uint4 *>(cu + i * M);
-        float acc = 0.f;
+        uint32_t words[M / 4];
 #pragma unroll
         for (int w = 0; w < M / 16; ++w) {
             const uint4 cw = cp[w];
-            const uint32_t words[4] = {cw.x, cw.y, cw.z, cw.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-#pragma unroll
-                for (int bb = 0; bb < 4; ++bb) {
-                    const int sub = w * 16 + k * 4 + bb;
-                    acc += s_lut[sub * 256 + ((words[k] >> (8 * bb)) & 0xffu)];
-                }
+            words[4 * w + 0] = cw.x;
+            words[4 * w + 1] = cw.y;
+            words[4 * w + 2] = cw.z;
+            words[4 * w + 3] = cw.w;
         }
+        const float acc = pq_adc_score<M>(words, s_lut, ln);
         su[i] = acc;
         if (hist) {
             uint32_t key, bucket;

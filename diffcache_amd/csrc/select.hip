@@ -213,10 +213,14 @@ __global__ __launch_bounds__(kFinalThreads) void sort_kernel(
         buf[i] = v;
     }
     __syncthreads();
+    // Pairs t in [64w, 64w + 64) (and the same range shifted by multiples of the block
+    // size) belong to wave w.  With a stride of at most 64 they lie inside the wave's own
+    // 128 elements, and a wave's LDS operations complete in order, so those stages need no
+    // block barrier: only the stages that cross waves, and the step into one, have one.
     for (int size = 2; size <= pow2; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int stride = size >> 1, ls = __ffs(size) - 2; stride > 0; stride >>= 1, --ls) {
             for (int t = tid; t < (pow2 >> 1); t += kFinalThreads) {
-                const int i = ((t / stride) * 2 * stride) + (t % stride);
+                const int i = ((t >> ls) << (ls + 1)) | (t & (stride - 1));
                 const int j = i + stride;
                 const bool asc = (i & size) == 0;
                 unsigned long long a = buf[i], b = buf[j];
@@ -225,9 +229,14 @@ __global__ __launch_bounds__(kFinalThreads) void sort_kernel(
                     buf[j] = a;
                 }
             }
-            __syncthreads();
+            if (!IN_LDS || stride > 64 || (stride == 1 && size >= 128)) __syncthreads();
+            else {
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // compiler ordering only
+                __builtin_amdgcn_wave_barrier();
+            }
         }
     }
+    __syncthreads();
     for (int i = tid; i < k_eff; i += kFinalThreads) io[i] = (uint32_t)(buf[i] & 0xffffffffull);
 }
 

@@ -67,11 +67,9 @@ class PQIndex:
         self.n_cand, self.topk = min(n_cand, n), min(topk, n)
         dev = store_k.device
         nu = b * h
-        self.hist = hip.new_hist(nu, dev)
-        self.cand = torch.empty((nu, self.n_cand), dtype=torch.int32, device=dev)
-        self.pos = torch.empty((nu, self.topk), dtype=torch.int32, device=dev)
-        self.ws1 = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, n, self.n_cand), dev)
-        self.ws2 = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, self.n_cand, self.topk), dev)
+        self.ids = torch.empty((nu, self.topk), dtype=torch.int32, device=dev)
+        self.ws = hip.alloc_workspace(hip.lib.dc_pq_search_workspace_bytes(nu, n, self.n_cand), dev)
+        self._ws_ready = False      # every search leaves the workspace ready for the next one
 
     @classmethod
     def build(cls, store_k: torch.Tensor, m: int = 32, sample: int = 65536, iters: int = 8,
@@ -83,13 +81,22 @@ class PQIndex:
         return cls(store_k, books, codes, **kw)
 
     def search(self, q: torch.Tensor) -> torch.Tensor:
-        """q (b*h, hd) bf16 -> int32 ids (b*h, topk), best exact score first."""
+        """q (b*h, hd) bf16 -> int32 ids (b*h, topk), best exact score first.  The returned
+        tensor is reused by the next call."""
         lut = hip.pq_build_lut(q, self.books, self.b)
-        self.hist.zero_()
-        adc = hip.pq_adc_scan(self.codes, lut, hist=self.hist)
-        cand = hip.topk_select(adc, self.n_cand, hip.MODE_IP, hip.ORDER_INDEX, hist=self.hist,
-                               idx_out=self.cand, workspace=self.ws1)
+        ids = hip.pq_search(self.store_k, self.codes, lut, q, self.n_cand, self.topk,
+                            idx_out=self.ids, workspace=self.ws, state_ready=self._ws_ready)
+        self._ws_ready = True
+        return ids
+
+    def search_stepwise(self, q: torch.Tensor) -> torch.Tensor:
+        """The same search through the separate entry points, with a dense ADC score array:
+        dc_pq_adc_scan -> dc_topk_select -> dc_score_gathered_bf16 -> dc_topk_select ->
+        dc_compose_idx.  Same ids as search()."""
+        lut = hip.pq_build_lut(q, self.books, self.b)
+        hist = hip.new_hist(self.b * self.h, q.device)
+        adc = hip.pq_adc_scan(self.codes, lut, hist=hist)
+        cand = hip.topk_select(adc, self.n_cand, hip.MODE_IP, hip.ORDER_INDEX, hist=hist)
         exact = hip.score_gathered(self.store_k, q, cand)
-        pos = hip.topk_select(exact, self.topk, hip.MODE_IP, hip.ORDER_BEST, idx_out=self.pos,
-                              workspace=self.ws2)
+        pos = hip.topk_select(exact, self.topk, hip.MODE_IP, hip.ORDER_BEST)
         return hip.compose_idx(cand, pos)

@@ -310,7 +310,9 @@ int dc_decode_layer(const dc_layer_args *args, void *stream);
  *   dc_pq_build_lut: lut[u, m, c] = q[u, m*ds:(m+1)*ds] . books[h(u), m, c, :]
  *     q (n_b*n_h, hd) bf16, books (n_h, M, 256, ds) fp32, lut (n_b*n_h, M, 256) fp32
  *   dc_pq_adc_scan: scores[u, i] = sum_m lut[u, m, codes[u, i, m]]
- *     codes (n_units, n_rows, M) uint8, fp32 adds in ascending m;
+ *     codes (n_units, n_rows, M) uint8; the fp32 adds of key i run over
+ *     m = i mod M, (i mod M) + 1, ... cyclically (the order that keeps the LDS
+ *     table reads of a wave in different banks);
  *     hist as in dc_score_bf16 (keys in DC_MODE_IP order), or NULL
  *   dc_score_gathered_bf16: scores[u, j] = q[u] . k[row_offset + idx[u, j]]  (exact rerank)
  *   dc_compose_idx: out[u, j] = outer[u, inner[u, j]]
@@ -326,6 +328,31 @@ int dc_score_gathered_bf16(const void *k, const void *q, const uint32_t *idx, fl
 int dc_compose_idx(const uint32_t *outer, int64_t outer_unit_stride, const uint32_t *inner,
                    int64_t inner_unit_stride, uint32_t *out, int64_t out_unit_stride, int n_units,
                    int n_inner, void *stream);
+
+/*
+ * The whole PQ search in one call, without a dense ADC score array:
+ *   candidates = the min(n_cand, n_rows) keys of every unit with the largest ADC
+ *                scores (ties to the lower id), scores as dc_pq_adc_scan computes them;
+ *   idx_out[u, 0 .. min(topk, n_rows)) = the candidates with the largest exact scores
+ *                q[u] . k[id] (as dc_score_gathered_bf16 computes them), best first,
+ *                ties to the lower id.
+ * Same ids as dc_pq_adc_scan -> dc_topk_select(DC_ORDER_INDEX) ->
+ * dc_score_gathered_bf16 -> dc_topk_select(DC_ORDER_BEST) -> dc_compose_idx.
+ * q (n_b*n_h, hd) bf16, lut from dc_pq_build_lut, codes (n_b*n_h, n_rows, M) uint8,
+ * k the bf16 key store with element strides; workspace from dc_pq_search_workspace_bytes.
+ * state_ready: 0 = the call initialises the selection state of the workspace itself;
+ * 1 = the previous call on this workspace was a dc_pq_search_bf16 with the same
+ * n_units, n_rows and n_cand and ran to completion (every call leaves the state ready).
+ * ev_scan_begin / ev_scan_end: optional hipEvent_t recorded on the stream around the
+ * scan kernel (NULL: none).
+ */
+size_t dc_pq_search_workspace_bytes(int n_units, int n_rows, int n_cand);
+int dc_pq_search_bf16(const void *k, const uint8_t *codes, const float *lut, const void *q,
+                      uint32_t *idx_out, int64_t idx_unit_stride, int n_b, int n_h, int n_rows,
+                      int hd, int m, int64_t k_batch_stride, int64_t k_head_stride,
+                      int64_t k_row_stride, int n_cand, int topk, int state_ready,
+                      void *workspace, size_t workspace_bytes, void *ev_scan_begin,
+                      void *ev_scan_end, void *stream);
 
 #ifdef __cplusplus
 }

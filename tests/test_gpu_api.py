@@ -493,6 +493,55 @@ def test_pq_index_search_matches_oracle_pipeline():
         assert len(true & set(ids[u].tolist())) >= 40      # recall of ADC with 1024 candidates
 
 
+@pytest.mark.parametrize("b,h,n,hd,m,n_cand,topk", [
+    (1, 2, 30000, 128, 32, 1024, 128),
+    (2, 3, 5000, 64, 16, 700, 100),      # 16 subspaces, ragged sizes
+    (1, 1, 300, 128, 32, 4096, 1024),    # fewer keys than candidates: everything is reranked
+    (1, 2, 70000, 256, 32, 9000, 5000),  # candidate list beyond the LDS staging of the finish kernel
+    (1, 1, 1, 128, 32, 4, 4),
+])
+def test_pq_search_fused_matches_stepwise(b, h, n, hd, m, n_cand, topk):
+    """dc_pq_search_bf16 (no dense ADC array) returns the ids of the entry-point chain
+    dc_pq_adc_scan -> dc_topk_select -> dc_score_gathered_bf16 -> dc_topk_select -> dc_compose_idx,
+    twice in a row on one workspace."""
+    from diffcache_amd.pq import PQIndex
+    rng = np.random.default_rng(n + m)
+    keys = rand_bf16(rng, b, h, n, hd)
+    store = dev_bf16(keys)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    books = torch.randn((h, m, 256, hd // m), generator=g, device=DEV)
+    codes = torch.randint(0, 256, (b * h, n, m), generator=g, device=DEV, dtype=torch.uint8)
+    index = PQIndex(store, books, codes, n_cand=n_cand, topk=topk)
+    for rep in range(2):
+        q = dev_bf16(rand_bf16(rng, b * h, hd))
+        want = index.search_stepwise(q).cpu().numpy()
+        got = index.search(q).cpu().numpy()
+        assert got.shape == want.shape == (b * h, min(topk, n))
+        assert np.array_equal(got, want), (rep, np.argwhere(got != want)[:4])
+
+
+def test_pq_search_fused_ties():
+    """Few distinct code rows and repeated key rows: ADC scores and exact scores tie in
+    large groups, and both stages must break ties to the lower id."""
+    from diffcache_amd.pq import PQIndex
+    rng = np.random.default_rng(77)
+    b, h, n, hd, m = 1, 2, 20000, 128, 32
+    base = rand_bf16(rng, 1, h, 7, hd)
+    pick = rng.integers(0, 7, n)
+    keys = np.ascontiguousarray(base[:, :, pick])
+    store = dev_bf16(keys)
+    g = torch.Generator(device=DEV).manual_seed(6)
+    books = torch.randn((h, m, 256, hd // m), generator=g, device=DEV)
+    rows = torch.randint(0, 256, (b * h, 5, m), generator=g, device=DEV, dtype=torch.uint8)
+    sel = torch.from_numpy(rng.integers(0, 5, n)).to(DEV)
+    codes = rows[:, sel].contiguous()
+    index = PQIndex(store, books, codes, n_cand=3000, topk=500)
+    q = dev_bf16(rand_bf16(rng, b * h, hd))
+    want = index.search_stepwise(q).cpu().numpy()
+    got = index.search(q).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 # ---------------------------------------------------------------- decode harness
 
 def test_harness_decode_step_matches_dense_attention():

@@ -96,6 +96,29 @@ def test_invalid_arguments_of_the_sketch_and_k_check_entry_points():
     assert rc == -22 and b"scores_unit_stride" in lib.dc_last_error()
 
 
+def test_invalid_arguments_of_the_pq_search_entry_point():
+    from diffcache_amd import _hip
+    lib = _hip.lib
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    # dc_pq_search_bf16(k, codes, lut, q, idx_out, idx_stride, n_b, n_h, n_rows, hd, m, k strides,
+    #                   n_cand, topk, state_ready, workspace, workspace_bytes, ev, ev, stream)
+    head = [p, p, p, p, p, 8, 1, 1, 64, 128]
+    rc = lib.dc_pq_search_bf16(*head, 24, 0, 0, 128, 16, 8, 0, p, 4096, None, None, None)
+    assert rc == -22 and b"subspaces" in lib.dc_last_error()
+    rc = lib.dc_pq_search_bf16(*head, 32, 0, 0, 128, 8, 16, 0, p, 4096, None, None, None)
+    assert rc == -22 and b"topk <= n_cand" in lib.dc_last_error()
+    rc = lib.dc_pq_search_bf16(*head, 32, 0, 0, 128, 16, 8, 0, p, 16, None, None, None)
+    assert rc == -12 and b"workspace" in lib.dc_last_error()
+    rc = lib.dc_pq_search_bf16(p, None, p, p, p, 8, 1, 1, 64, 128, 32, 0, 0, 128, 16, 8, 0, p, 4096, None,
+                               None, None)
+    assert rc == -22 and b"null pointer" in lib.dc_last_error()
+    # nothing to do: no rows, or no results wanted
+    assert lib.dc_pq_search_bf16(p, p, p, p, p, 8, 1, 1, 0, 128, 32, 0, 0, 128, 16, 8, 0, None, 0, None,
+                                 None, None) == 0
+    assert lib.dc_pq_search_workspace_bytes(8, 1000, 64) > lib.dc_score_select_workspace_bytes(8, 1000, 64)
+
+
 def test_data_layer_option_errors():
     from diffcache_amd import DiffCacheHIP
     from diffcache_amd._hip import DiffCacheError
