@@ -34,6 +34,8 @@ k_check_budget         the epoch loop of nsw.rs:302-303,339,367-379 applied to
 pq_*                   no reference source (evaluation/impl/pqcache is an
                        empty directory): PARITY UNPINNED at the reference;
                        pinned by closed forms in tests/test_oracle_pq.py
+                       (pq_adc_scores_f32 restates the HIP kernels' documented
+                       fp32 order of additions and is compared bit for bit)
 =====================  =====================================================
 
 Parity status.  The reference holds golden vectors only for ``DualHeap``
@@ -437,6 +439,19 @@ def pq_adc_scores(codes: np.ndarray, lut: np.ndarray) -> np.ndarray:
     """s_i = sum_m LUT[m][codes[i, m]], float64."""
     m = lut.shape[0]
     return lut[np.arange(m)[None, :], codes.astype(np.int64)].sum(axis=1)
+
+
+def pq_adc_scores_f32(codes: np.ndarray, lut_f32: np.ndarray) -> np.ndarray:
+    """The same sums in fp32 and in the order the HIP kernels document: key i adds
+    subspaces (i mod M), (i mod M) + 1, ... cyclically, starting from 0.0f."""
+    n, m = codes.shape
+    lut_f32 = lut_f32.astype(np.float32)
+    rows = np.arange(n)
+    acc = np.zeros(n, dtype=np.float32)
+    for j in range(m):
+        s = (rows + j) % m
+        acc = (acc + lut_f32[s, codes[rows, s].astype(np.int64)]).astype(np.float32)
+    return acc
 
 
 def pq_reconstruct(codes: np.ndarray, books: np.ndarray) -> np.ndarray:

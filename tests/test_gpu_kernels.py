@@ -777,6 +777,8 @@ def test_pq_lut_scan_and_rerank():
     for h in range(n_h):
         want = orc.pq_adc_scores(codes[h], lut_np[h].astype(np.float64))
         assert np.allclose(adc_np[h], want, rtol=1e-5, atol=1e-4)
+        # bit for bit with the fp32 restatement of the documented order of additions
+        assert np.array_equal(adc_np[h], orc.pq_adc_scores_f32(codes[h], lut_np[h]))
         assert np.array_equal(hist.cpu().numpy()[h],
                               np.bincount(orc.coarse_bucket(adc_np[h], 0), minlength=hip.HIST_BINS))
     n_cand, topk = 2048, 256

@@ -65,3 +65,28 @@ def test_pq_search_rerank_is_exact_topk_of_candidates():
     # recall of the true top-50 inside 400 ADC candidates is high on Gaussian data
     true = set(orc.topk_select(s, 50, orc.MODE_IP).tolist())
     assert len(true & set(top.tolist())) >= 35
+
+
+def test_pq_adc_fp32_order_agrees_with_float64_sum():
+    """The fp32 restatement (cyclic order of additions) stays within fp32 rounding of the
+    float64 sum, and is that sum exactly when the table holds small integers."""
+    rng = np.random.default_rng(3)
+    n, m = 3000, 32
+    codes = rng.integers(0, 256, (n, m), dtype=np.uint8)
+    lut = rng.standard_normal((m, 256)).astype(np.float32)
+    want = orc.pq_adc_scores(codes, lut.astype(np.float64))
+    got = orc.pq_adc_scores_f32(codes, lut)
+    assert got.dtype == np.float32
+    assert np.max(np.abs(got - want)) <= 32 * 2.0 ** -23 * np.abs(lut).max() * m
+    lut_i = rng.integers(-1000, 1000, (m, 256)).astype(np.float32)
+    assert np.array_equal(orc.pq_adc_scores_f32(codes, lut_i),
+                          orc.pq_adc_scores(codes, lut_i.astype(np.float64)).astype(np.float32))
+    # 16 subspaces, key i starts from subspace i mod 16: one key, spelled out
+    lut16 = rng.standard_normal((16, 256)).astype(np.float32)
+    c16 = rng.integers(0, 256, (40, 16), dtype=np.uint8)
+    i = 37
+    acc = np.float32(0)
+    for j in range(16):
+        sub = (i + j) % 16
+        acc = np.float32(acc + lut16[sub, c16[i, sub]])
+    assert orc.pq_adc_scores_f32(c16, lut16)[i] == acc
