@@ -359,13 +359,17 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
     const unsigned long long lt = (1ull << lane) - 1ull;
 
     // Double buffering: the loads of the next step are issued before the current step is
-    // worked on, so a wave always has a step's worth of bytes in flight.
+    // worked on, so a wave always has a step's worth of bytes in flight.  The loads are
+    // unconditional (past the block's end they repeat its last row), which lets the
+    // compiler wait for exactly the older buffer instead of for every load in flight.
+    const int64_t blk_end = block_row0 + (int64_t)steps * kRowsPerBlockStep - 1;
+    const int64_t blk_last = blk_end < (int64_t)last ? blk_end : (int64_t)last;
     auto load_step = [&](int step, uint4 (&cv)[LPR]) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
 #pragma unroll
         for (int j = 0; j < LPR; ++j) {
             int64_t r = row0 + grp * LPR + j;
-            r = r > last ? last : r;
+            r = r > blk_last ? blk_last : r;
             cv[j] = *reinterpret_cast<const uint4 *>(Cu + r * cr);
         }
     };
@@ -397,21 +401,21 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
         }
     }
     uint4 ca[LPR], cb2[LPR];
-    if (my_steps > 0) load_step(0, ca);
+    load_step(0, ca);
     // The threshold poll is issued before the prefetch: loads return in order, so waiting
     // for a poll that was issued last would also wait for the whole prefetch.
-    for (int step = 0; step < my_steps; step += 2) {
+    int step = 0;
+    for (; step + 1 < my_steps; step += 2) {
         uint32_t tb_next = load_relaxed(&st->tb_run);
-        if (step + 1 < my_steps) load_step(step + 1, cb2);
+        load_step(step + 1, cb2);
         work_step(step, ca);
         tb = tb_next;
-        if (step + 1 < my_steps) {
-            tb_next = load_relaxed(&st->tb_run);
-            if (step + 2 < my_steps) load_step(step + 2, ca);
-            work_step(step + 1, cb2);
-            tb = tb_next;
-        }
+        tb_next = load_relaxed(&st->tb_run);
+        load_step(step + 2, ca);
+        work_step(step + 1, cb2);
+        tb = tb_next;
     }
+    if (step < my_steps) work_step(step, ca);  // an odd last step; its rows are already on the way
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
                        surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
