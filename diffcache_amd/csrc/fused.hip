@@ -958,8 +958,13 @@ int plan_fused(const char *who, int n_b, int n_h, int n_rows, int budget, FusedP
     DC_REQUIRE(n_units64 < (1 << 20), "%s: too many units", who);
     p->n_units = (int)n_units64;
     p->k_eff = budget < n_rows ? budget : n_rows;
-    // chunks per unit: up to kSmallChunks blocks of one step, then blocks of big_steps steps
+    // chunks per unit: up to kSmallChunks blocks of one step, then blocks of big_steps steps.
+    // Short scans take fewer steps per block so that the grid still has a few thousand
+    // blocks: a block's steps run one after the other, and with few blocks the kernel
+    // lasts as long as its longest block.
     const int64_t tiles = ((int64_t)n_rows + rows_per_step - 1) / rows_per_step;
+    const int64_t fill = n_units64 * tiles / 2048;
+    if (fill < big_steps) big_steps = fill < 1 ? 1 : (int)fill;
     p->big_steps = big_steps;
     p->small_chunks = (int)(tiles < kSmallChunks ? tiles : kSmallChunks);
     const int64_t rest = (int64_t)n_rows - (int64_t)p->small_chunks * rows_per_step;
