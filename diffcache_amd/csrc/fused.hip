@@ -216,7 +216,7 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
             for (int j = 0; j < CH; ++j) {
                 int64_t r = row0 + grp * LPR + c0 + j;
                 r = r > last ? last : r;
-                w[j] = *reinterpret_cast<const uint4 *>(Ku + r * sr);
+                w[j] = dc_load_stream16(Ku + r * sr);
             }
             // the threshold for the next step queues up behind this step's rows
             if (c0 + CH >= LPR && step + 1 < steps) tb_next = load_relaxed(&st->tb_run);
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
         for (int j = 0; j < LPR; ++j) {
             int64_t r = row0 + grp * LPR + j;
             r = r > blk_last ? blk_last : r;
-            cv[j] = *reinterpret_cast<const uint4 *>(Cu + r * cr);
+            cv[j] = dc_load_stream16(Cu + r * cr);
         }
     };
     auto work_step = [&](int step, const uint4 (&cv)[LPR]) {
@@ -465,6 +465,7 @@ __global__ __launch_bounds__(kPqThreads) void pq_prune_kernel(
     auto load_row = [&](int64_t row0, uint32_t(&w)[NW]) {
         int64_t r = row0 + lane;
         r = r > blk_last ? blk_last : r;
+        // plain loads: the two halves of a 32-byte row come from the same cache line
         const uint4 *cp = reinterpret_cast<const uint4 *>(cu + r * M);
 #pragma unroll
         for (int i = 0; i < NW / 4; ++i) {

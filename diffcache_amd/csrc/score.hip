@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
             for (int j = 0; j < CH; ++j) {
                 int64_t r = row0 + grp * LPR + c0 + j;
                 r = r > last ? last : r;  // keep the load in bounds; masked below
-                w[j] = *reinterpret_cast<const uint4 *>(Ku + r * sr);
+                w[j] = dc_load_stream16(Ku + r * sr);
             }
 #pragma unroll
             for (int j = 0; j < CH; ++j) {

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kThreads) void sketch_absmax_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) m[i] = 0;
     for (int64_t r = r0 + grp; r < r1; r += GROUPS) {
-        const uint4 w = *reinterpret_cast<const uint4 *>(Ku + r * sr);
+        const uint4 w = dc_load_stream16(Ku + r * sr);
         const uint32_t x[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void sketch_quantise_kernel(
     int64_t r1 = r0 + kRowsPerBlock;
     if (r1 > n_rows) r1 = n_rows;
     for (int64_t r = r0 + grp; r < r1; r += GROUPS) {
-        const uint4 w = *reinterpret_cast<const uint4 *>(Ku + r * sr);
+        const uint4 w = dc_load_stream16(Ku + r * sr);
         const float kv[8] = {dc_bf16_lo(w.x), dc_bf16_hi(w.x), dc_bf16_lo(w.y), dc_bf16_hi(w.y),
                              dc_bf16_lo(w.z), dc_bf16_hi(w.z), dc_bf16_lo(w.w), dc_bf16_hi(w.w)};
         uint32_t code[8];
