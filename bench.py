@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes one scan launch of config 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE scaled
 # by a known-size copy kernel (the figures and commands are kept with the other profile
 # summaries of this repository): counts x 2 KiB read + counts x 1 KiB written.
-SCAN_TRAFFIC_BYTES_C3 = {"sketch": 525_700 * 2048 + 13_577 * 1024,
+SCAN_TRAFFIC_BYTES_C3 = {"sketch": 524_722 * 2048 + 13_249 * 1024,
                          "bf16": 1_053_933 * 2048 + 12_570 * 1024}
 
 CONFIGS = {
