@@ -47,6 +47,18 @@ __device__ __forceinline__ uint4 dc_load_stream16(const void *p) {
     return make_uint4(t.x, t.y, t.z, t.w);
 }
 
+// the matching stores, for bulk data that the writing kernel does not read back
+__device__ __forceinline__ void dc_store_stream16(void *p, uint4 v) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(p));
+}
+__device__ __forceinline__ void dc_store_stream8(void *p, uint2 v) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 t = {v.x, v.y};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x2 *>(p));
+}
+
 __device__ __forceinline__ float dc_bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float dc_bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 __device__ __forceinline__ float dc_bf16_to_f32(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }

@@ -39,7 +39,7 @@ __global__ void ingest_kernel(uint16_t *__restrict__ store, const uint16_t *__re
     const int64_t s = r % seq;
     const int64_t b = r / seq;
     const int64_t dst = b * sb + h * sh + (dst_pos + s) * sr + c * 8;
-    *reinterpret_cast<uint4 *>(store + dst) = dc_load_stream16(src + t * 8);
+    dc_store_stream16(store + dst, dc_load_stream16(src + t * 8));
 }
 
 }  // namespace

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void sketch_quantise_kernel(
         uint2 packed;
         packed.x = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
         packed.y = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
-        *reinterpret_cast<uint2 *>(Cu + r * cr) = packed;
+        dc_store_stream8(Cu + r * cr, packed);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) smax[grp][col * 8 + i] = __float_as_uint(res[i]);
