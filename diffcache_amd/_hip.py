@@ -35,6 +35,8 @@ SYMBOLS = (
     "dc_sketch_build_bf16", "dc_sketch_select_workspace_bytes", "dc_sketch_select_state_init",
     "dc_score_select_sketch_bf16", "dc_kcheck_f32",
     "dc_pq_search_workspace_bytes", "dc_pq_search_bf16",
+    "dc_data_layer_create", "dc_data_layer_destroy", "dc_data_layer_ctx_len", "dc_data_layer_sizes",
+    "dc_data_layer_bind", "dc_data_layer_prefill", "dc_data_layer_insert", "dc_data_layer_query",
 )
 
 
@@ -86,6 +88,14 @@ def _load() -> C.CDLL:
         "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
         "dc_compose_idx": (i, [p, i64, p, i64, p, i64, i, i, p]),
         "dc_pq_search_workspace_bytes": (sz, [i, i, i]),
+        "dc_data_layer_create": (i, [C.POINTER(p), i, i, i, i64, i, i]),
+        "dc_data_layer_destroy": (None, [p]),
+        "dc_data_layer_ctx_len": (i64, [p]),
+        "dc_data_layer_sizes": (i, [p, i] + [C.POINTER(sz)] * 5),
+        "dc_data_layer_bind": (i, [p, p, p, p, p, p, p, p, sz, i]),
+        "dc_data_layer_prefill": (i, [p, p, p, i64, p]),
+        "dc_data_layer_insert": (i, [p, p, p, p]),
+        "dc_data_layer_query": (i, [p, p, p, i64, p, i, C.POINTER(i), p]),
         "dc_pq_search_bf16": (i, [p, p, p, p, p, i64, i, i, i, i, i, i64, i64, i64, i, i, i, p, sz, p, p, p]),
         "dc_score_select_workspace_bytes": (sz, [i, i, i]),
         "dc_select_state_init": (i, [i, i, i, p, sz, p]),

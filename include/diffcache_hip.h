@@ -354,6 +354,43 @@ int dc_pq_search_bf16(const void *k, const uint8_t *codes, const float *lut, con
                       void *workspace, size_t workspace_bytes, void *ev_scan_begin,
                       void *ev_scan_end, void *stream);
 
+/*
+ * The reference's data layer as a handle (struct DataLayer, diffcache_cpu/src/lib.rs:189-197):
+ * shape, capacity and context length on the host, over device buffers the caller owns.
+ * For hosts that are not Python (the Python mirror is diffcache_amd.DiffCacheHIP).
+ *   create   DataLayer::new, lib.rs:292-327.  mode: DC_MODE_*; use_sketch: keep the 8-bit
+ *            sketch of the keys and query through it (same results).
+ *   sizes    bytes of the buffers to bind: store_bytes for EACH of the K and V stores
+ *            (bsz, kv_heads, max_ctx_len, hd) bf16, codes_bytes, scale_bytes for EACH of
+ *            scale and resid (0 without the sketch), idx_bytes, workspace_bytes; max_ef =
+ *            the largest ef a query will ask for.
+ *   bind     hands the buffers over (16-byte aligned, the workspace 256-byte aligned).
+ *   prefill  lib.rs:329-347: keys, vals (bsz, kv_heads, n_rows, hd) bf16 in host or device
+ *            memory replace the contents; n_rows <= max_ctx_len.
+ *   insert   lib.rs:352-369: keys, vals (bsz, kv_heads, hd) bf16 in device memory, one
+ *            token per unit, appended at ctx_len; an error when the store is full.
+ *   query    lib.rs:373-404 with nsw.rs:592-630: queries (bsz, kv_heads, hd) bf16; the
+ *            min(ef, ctx_len) best K and V rows of every unit, best first, ties to the
+ *            lower id, into out_keys / out_vals (bsz, kv_heads, out_rows, hd) in device
+ *            memory; *n_out (may be NULL) = rows written per unit.
+ * prefill, insert and query only enqueue work on `stream`; calls on one handle must not
+ * overlap.  destroy frees the handle, never the buffers.
+ */
+typedef struct dc_data_layer dc_data_layer;
+int dc_data_layer_create(dc_data_layer **out, int bsz, int kv_heads, int hd, int64_t max_ctx_len,
+                         int mode, int use_sketch);
+void dc_data_layer_destroy(dc_data_layer *dl);
+int64_t dc_data_layer_ctx_len(const dc_data_layer *dl);
+int dc_data_layer_sizes(const dc_data_layer *dl, int max_ef, size_t *store_bytes, size_t *codes_bytes,
+                        size_t *scale_bytes, size_t *idx_bytes, size_t *workspace_bytes);
+int dc_data_layer_bind(dc_data_layer *dl, void *k_store, void *v_store, void *codes, void *scale,
+                       void *resid, void *idx, void *workspace, size_t workspace_bytes, int max_ef);
+int dc_data_layer_prefill(dc_data_layer *dl, const void *keys, const void *vals, int64_t n_rows,
+                          void *stream);
+int dc_data_layer_insert(dc_data_layer *dl, const void *keys, const void *vals, void *stream);
+int dc_data_layer_query(dc_data_layer *dl, void *out_keys, void *out_vals, int64_t out_rows,
+                        const void *queries, int ef, int *n_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -458,6 +458,86 @@ def test_diffcache_prefill_cache_roundtrip(tmp_path):
     assert np.array_equal(outs[0], outs[1])
 
 
+# ---------------------------------------------------------------- the C handle of the data layer
+
+@pytest.mark.parametrize("use_sketch", [False, True])
+def test_c_data_layer_matches_python_data_layer(use_sketch):
+    """dc_data_layer_* (the C++ host mirror of lib.rs:189-404) driven through ctypes: prefill,
+    a few inserts and queries give the rows DiffCacheHIP gives, which the other tests check
+    against the oracle; ef larger than the context is clamped (lib.rs:374)."""
+    import ctypes
+    from diffcache_amd import DiffCacheHIP, _hip
+    lib = _hip.lib
+    rng = np.random.default_rng(31)
+    b, hq, hkv, hd, n_max, n0, max_ef = 2, 8, 2, 128, 700, 600, 96
+    keys, vals = rand_bf16(rng, b, hkv, n0, hd), rand_bf16(rng, b, hkv, n0, hd)
+    ref = DiffCacheHIP(b, hq, hkv, hd, max_ctx_len=n_max, key_sketch=use_sketch)
+    ref.prefill(keys, vals)
+
+    h = ctypes.c_void_p()
+    assert lib.dc_data_layer_create(ctypes.byref(h), b, hkv, hd, n_max, _hip.MODE_REF_DIST, int(use_sketch)) == 0
+    try:
+        sz = [ctypes.c_size_t() for _ in range(5)]
+        assert lib.dc_data_layer_sizes(h, max_ef, *[ctypes.byref(x) for x in sz]) == 0
+        store_b, codes_b, scale_b, idx_b, ws_b = [x.value for x in sz]
+        kst = torch.zeros(store_b // 2, dtype=torch.bfloat16, device=DEV)
+        vst = torch.zeros(store_b // 2, dtype=torch.bfloat16, device=DEV)
+        codes = torch.zeros(max(codes_b, 16), dtype=torch.uint8, device=DEV)
+        scale = torch.zeros(max(scale_b // 4, 4), dtype=torch.float32, device=DEV)
+        resid = torch.zeros(max(scale_b // 4, 4), dtype=torch.float32, device=DEV)
+        idx = torch.zeros(idx_b // 4, dtype=torch.int32, device=DEV)
+        ws = _hip.alloc_workspace(ws_b, DEV)
+        sk = (codes.data_ptr(), scale.data_ptr(), resid.data_ptr()) if use_sketch else (None, None, None)
+        assert lib.dc_data_layer_bind(h, kst.data_ptr(), vst.data_ptr(), *sk, idx.data_ptr(), ws.data_ptr(),
+                                      ws.numel() * ws.element_size(), max_ef) == 0
+        stream = torch.cuda.current_stream().cuda_stream
+        # prefill from host memory, as the pyo3 class takes it
+        kh, vh = np.ascontiguousarray(keys), np.ascontiguousarray(vals)
+        assert lib.dc_data_layer_prefill(h, kh.ctypes.data, vh.ctypes.data, n0, stream) == 0, lib.dc_last_error()
+        torch.cuda.synchronize()
+        assert lib.dc_data_layer_ctx_len(h) == n0
+
+        def query(ef):
+            q = rand_bf16(rng, b, hkv, hd)
+            want_k = torch.zeros((b, hkv, max_ef, hd), dtype=torch.bfloat16, device=DEV)
+            want_v = torch.zeros_like(want_k)
+            ref.query(want_k, want_v, q, ef)
+            got_k, got_v = torch.zeros_like(want_k), torch.zeros_like(want_k)
+            qd = dev_bf16(q)
+            n_out = ctypes.c_int(-1)
+            rc = lib.dc_data_layer_query(h, got_k.data_ptr(), got_v.data_ptr(), max_ef, qd.data_ptr(), ef,
+                                         ctypes.byref(n_out), stream)
+            assert rc == 0, lib.dc_last_error()
+            torch.cuda.synchronize()
+            assert n_out.value == min(ef, ref.ctx_len)
+            assert torch.equal(got_k.view(torch.int16), want_k.view(torch.int16))
+            assert torch.equal(got_v.view(torch.int16), want_v.view(torch.int16))
+
+        query(64)
+        for _ in range(5):       # rows outside the fitted range of the sketch included
+            nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+            nk[0, 0, :4] = orc.f32_to_bf16(np.array([40.0, -35.0, 20.0, 9.0], dtype=np.float32))
+            ref.insert(nk, nv)
+            assert lib.dc_data_layer_insert(h, dev_bf16(nk).data_ptr(), dev_bf16(nv).data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+        assert lib.dc_data_layer_ctx_len(h) == n0 + 5
+        query(96)
+        query(1)
+        # a tiny context: ef is clamped to it
+        assert lib.dc_data_layer_prefill(h, kh.ctypes.data, vh.ctypes.data, 0, stream) == 0
+        ref.ctx_len = 0
+        for _ in range(3):
+            nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+            ref.insert(nk, nv)
+            assert lib.dc_data_layer_insert(h, dev_bf16(nk).data_ptr(), dev_bf16(nv).data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+        query(64)
+        assert lib.dc_data_layer_query(h, kst.data_ptr(), vst.data_ptr(), max_ef, kst.data_ptr(), max_ef + 1,
+                                       None, stream) == -22
+    finally:
+        lib.dc_data_layer_destroy(h)
+
+
 # ---------------------------------------------------------------- PQ baseline
 
 def test_pq_index_search_matches_oracle_pipeline():

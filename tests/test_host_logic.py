@@ -119,6 +119,39 @@ def test_invalid_arguments_of_the_pq_search_entry_point():
     assert lib.dc_pq_search_workspace_bytes(8, 1000, 64) > lib.dc_score_select_workspace_bytes(8, 1000, 64)
 
 
+def test_c_data_layer_handle_bookkeeping_and_errors():
+    """dc_data_layer_*: the host-side mirror of lib.rs:189-404 as a C handle; everything that
+    needs no GPU (creation, sizes, argument checks)."""
+    from diffcache_amd import _hip
+    lib = _hip.lib
+    h = ctypes.c_void_p()
+    assert lib.dc_data_layer_create(ctypes.byref(h), 2, 4, 96, 1000, 1, 1) == -22
+    assert b"head_dim" in lib.dc_last_error() and not h.value
+    assert lib.dc_data_layer_create(ctypes.byref(h), 2, 4, 128, 1000, 7, 1) == -22
+    assert b"mode" in lib.dc_last_error()
+    assert lib.dc_data_layer_create(ctypes.byref(h), 2, 4, 128, 1000, 1, 1) == 0 and h.value
+    assert lib.dc_data_layer_ctx_len(h) == 0
+    sizes = [ctypes.c_size_t() for _ in range(5)]
+    assert lib.dc_data_layer_sizes(h, 64, *[ctypes.byref(x) for x in sizes]) == 0
+    store, codes, scale, idx, ws = [x.value for x in sizes]
+    assert store == 2 * 4 * 1000 * 128 * 2 and codes == 2 * 4 * 1000 * 128
+    assert scale == 2 * 4 * 128 * 4 and idx == 2 * 4 * 64 * 4
+    assert ws == lib.dc_sketch_select_workspace_bytes(8, 1000, 64)
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    # not bound yet
+    assert lib.dc_data_layer_prefill(h, p, p, 10, None) == -22 and b"bound" in lib.dc_last_error()
+    assert lib.dc_data_layer_insert(h, p, p, None) == -22
+    assert lib.dc_data_layer_query(h, p, p, 8, p, 8, None, None) == -22
+    # binding: missing sketch buffers, small workspace
+    assert lib.dc_data_layer_bind(h, p, p, None, None, None, p, p, ws, 64) == -22
+    assert b"sketch buffers" in lib.dc_last_error()
+    assert lib.dc_data_layer_bind(h, p, p, p, p, p, p, p, 16, 64) == -12
+    lib.dc_data_layer_destroy(h)
+    lib.dc_data_layer_destroy(None)
+    assert lib.dc_data_layer_ctx_len(None) == -1
+
+
 def test_data_layer_option_errors():
     from diffcache_amd import DiffCacheHIP
     from diffcache_amd._hip import DiffCacheError
