@@ -752,6 +752,39 @@ def test_decode_layer_config2_shape():
     run_layer(rng, 1, 32, 8, 32768, 128, 1024, 4, 64, hip.MODE_REF_DIST, True, k_scale=scale)
 
 
+@pytest.mark.parametrize("route", ["dense", "stream", "sketch"])
+def test_config1_planted_keys(route):
+    """Benchmark configuration 1, the reference's own CPU-runnable case: one KV head, N 8192,
+    hd 128, 16 planted keys = 3 q + 0.1 noise, k 256, no sinks, no recent window.  The planted
+    keys are the 16 best; the ids are those of the C restatement of search_bruteforce; the
+    output is the softmax-weighted sum of the selected V rows."""
+    from oracle import cpu_ref
+    rng = np.random.default_rng(1000)
+    n, hd, k = 8192, 128, 256
+    qf = rng.standard_normal(hd).astype(np.float32)
+    kf = rng.standard_normal((n, hd)).astype(np.float32)
+    planted = rng.choice(n, 16, replace=False)
+    kf[planted] = 3 * qf + 0.1 * rng.standard_normal((16, hd)).astype(np.float32)
+    q, keys, vals = orc.f32_to_bf16(qf), orc.f32_to_bf16(kf), rand_bf16(rng, n, hd)
+    _, _, want_ids, _ = cpu_ref.search_bruteforce(keys, vals, q, k)
+    store_k, store_v = to_dev_bf16(keys[None, None]), to_dev_bf16(vals[None, None])
+    qd = to_dev_bf16(q[None, None])                       # (b 1, heads 1, hd)
+    idx = torch.empty((1, k), dtype=torch.int32, device=DEV)
+    out = torch.empty((1, 1, hd), dtype=torch.bfloat16, device=DEV)
+    ws = hip.alloc_workspace(hip.layer_workspace_bytes(1, n, k, 1, hd, k), DEV)
+    scores = torch.empty((1, n), dtype=torch.float32, device=DEV) if route == "dense" else None
+    sketch = hip.Sketch(store_k).build(store_k, 0, n) if route == "sketch" else None
+    hip.decode_layer(qd, store_k, store_v, 0, n, 0, k, scores, idx, out, ws, None, None,
+                     mode=hip.MODE_REF_DIST, order=hip.ORDER_BEST, sketch=sketch)
+    torch.cuda.synchronize()
+    ids = idx.cpu().numpy()[0].astype(np.uint32)
+    assert set(ids[:16].tolist()) == set(planted.tolist())
+    assert np.array_equal(ids, want_ids)
+    res = orc.decode_layer(q[None], keys[None], vals[None], 1, k, 0, 0, orc.MODE_REF_DIST)
+    assert np.array_equal(ids, res["sel"][0])
+    assert bf16_close(orc.bf16_to_f32(to_np_u16(out))[0], res["out"])
+
+
 def test_decode_layer_qwen_shape_group7():
     run_layer(np.random.default_rng(70), 1, 28, 4, 5000, 128, 1024, 128, 128, hip.MODE_IP, True)
 
