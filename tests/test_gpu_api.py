@@ -579,6 +579,7 @@ def test_pq_index_search_matches_oracle_pipeline():
     (1, 1, 300, 128, 32, 4096, 1024),    # fewer keys than candidates: everything is reranked
     (1, 2, 70000, 256, 32, 9000, 5000),  # candidate list beyond the LDS staging of the finish kernel
     (1, 1, 1, 128, 32, 4, 4),
+    (1, 8, 1 << 20, 128, 32, 4096, 1024),   # benchmark configuration 4 at full size
 ])
 def test_pq_search_fused_matches_stepwise(b, h, n, hd, m, n_cand, topk):
     """dc_pq_search_bf16 (no dense ADC array) returns the ids of the entry-point chain
@@ -586,9 +587,8 @@ def test_pq_search_fused_matches_stepwise(b, h, n, hd, m, n_cand, topk):
     twice in a row on one workspace."""
     from diffcache_amd.pq import PQIndex
     rng = np.random.default_rng(n + m)
-    keys = rand_bf16(rng, b, h, n, hd)
-    store = dev_bf16(keys)
     g = torch.Generator(device=DEV).manual_seed(5)
+    store = torch.randn((b, h, n, hd), generator=g, device=DEV).to(torch.bfloat16)
     books = torch.randn((h, m, 256, hd // m), generator=g, device=DEV)
     codes = torch.randint(0, 256, (b * h, n, m), generator=g, device=DEV, dtype=torch.uint8)
     index = PQIndex(store, books, codes, n_cand=n_cand, topk=topk)
