@@ -337,12 +337,17 @@ int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t 
         // the ids are distinct and below n_rows: mark and sweep beats a bitonic sort
         const int n_words = (n_rows + 31) / 32;
         const size_t lds = (size_t)(n_words + (n_words >> 5) + 1) * 4;
-        static bool attr_set = false;
-        if (!attr_set) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(index_order_kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (kBitmapMaxRows / 32 + kBitmapMaxRows / 1024 + 1) * 4);
-            attr_set = true;
+        // more than the default 64 KB of dynamic LDS has to be asked for; the attribute
+        // belongs to the current device, so it is set on every such call (a host-side
+        // store), always to the same value so that concurrent callers cannot undercut it
+        if (lds > 64 * 1024) {
+            constexpr int kMaxLds = (kBitmapMaxRows / 32 + kBitmapMaxRows / 1024 + 1) * 4;
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(index_order_kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+            if (e != hipSuccess) {
+                dc_set_error("dc_sort_selected: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+                return DC_ELAUNCH;
+            }
         }
         hipLaunchKernelGGL(index_order_kernel, dim3(n_units), dim3(kFinalThreads), lds, st, idx_out,
                            idx_stride, k_eff, n_words);
