@@ -342,7 +342,8 @@ int dc_compose_idx(const uint32_t *outer, int64_t outer_unit_stride, const uint3
  * k the bf16 key store with element strides; workspace from dc_pq_search_workspace_bytes.
  * state_ready: 0 = the call initialises the selection state of the workspace itself;
  * 1 = the previous call on this workspace was a dc_pq_search_bf16 with the same
- * n_units, n_rows and n_cand and ran to completion (every call leaves the state ready).
+ * n_units, n_rows and n_cand, returned 0 and had work to do (n_rows > 0, topk > 0):
+ * every such call leaves the state ready for the next.
  * ev_scan_begin / ev_scan_end: optional hipEvent_t recorded on the stream around the
  * scan kernel (NULL: none).
  */
