@@ -149,6 +149,14 @@ def _store_strides(store: torch.Tensor) -> Tuple[int, int, int]:
     return store.stride(0), store.stride(1), store.stride(2)
 
 
+def require(cond: bool, msg: str = "") -> None:
+    """The reference asserts its invariants (Rust ``assert!`` -> a panic, Python ``assert``).
+    Here they guard device memory, so they must survive ``python -O``: same exception type,
+    not an ``assert`` statement."""
+    if not cond:
+        raise AssertionError(msg)
+
+
 def alloc_workspace(nbytes: int, device) -> torch.Tensor:
     """Zero-filled, 256-byte aligned scratch (the attention counters must start at zero)."""
     return torch.zeros((max(int(nbytes), 256) + 255) // 256 * 256, dtype=torch.uint8, device=device)

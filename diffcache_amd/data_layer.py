@@ -115,8 +115,8 @@ class DiffCacheHIP:
             # rows of an existing HBM store, e.g. the retrieval region of a layer's K/V
             self.keys, self.vals = storage
             want = (bsz, kv_head_num, self.max_ctx_len, head_dim)
-            assert tuple(self.keys.shape) == want and tuple(self.vals.shape) == want, \
-                f"storage must be two {want} bf16 tensors"
+            hip.require(tuple(self.keys.shape) == want and tuple(self.vals.shape) == want,
+                        f"storage must be two {want} bf16 tensors")
         self._ws: Optional[torch.Tensor] = None
         self._ws_key = None
         self._idx: Optional[torch.Tensor] = None
@@ -136,9 +136,9 @@ class DiffCacheHIP:
         v = _as_bf16(vals, self.device)
         seq = k.shape[2] if k.dim() == 4 else -1
         want = (self.bsz, self.kv_head_num, seq, self.head_dim)
-        assert tuple(k.shape) == want, f"keys shape {tuple(k.shape)} != {want}"        # lib.rs:332
-        assert tuple(v.shape) == want, f"vals shape {tuple(v.shape)} != {want}"        # lib.rs:333
-        assert seq <= self.max_ctx_len, "sequence longer than max_ctx_len"
+        hip.require(tuple(k.shape) == want, f"keys shape {tuple(k.shape)} != {want}")        # lib.rs:332
+        hip.require(tuple(v.shape) == want, f"vals shape {tuple(v.shape)} != {want}")        # lib.rs:333
+        hip.require(seq <= self.max_ctx_len, "sequence longer than max_ctx_len")
         self.keys[:, :, :seq].copy_(k)
         self.vals[:, :, :seq].copy_(v)
         self.ctx_len = seq
@@ -148,7 +148,7 @@ class DiffCacheHIP:
         """Ingest straight from the model layout (bsz, seq, kv_heads, hd) with the
         layout-transform kernel (what diffcache.py:142-147 does through the host)."""
         seq = key_states.shape[1]
-        assert seq <= self.max_ctx_len, "sequence longer than max_ctx_len"
+        hip.require(seq <= self.max_ctx_len, "sequence longer than max_ctx_len")
         hip.ingest_kv(self.keys, key_states, 0)
         hip.ingest_kv(self.vals, value_states, 0)
         self.ctx_len = seq
@@ -159,9 +159,9 @@ class DiffCacheHIP:
         k = _as_bf16(keys, self.device)
         v = _as_bf16(vals, self.device)
         want = (self.bsz, self.kv_head_num, self.head_dim)
-        assert tuple(k.shape) == want, f"keys shape {tuple(k.shape)} != {want}"        # lib.rs:353
-        assert tuple(v.shape) == want, f"vals shape {tuple(v.shape)} != {want}"        # lib.rs:354
-        assert self.ctx_len < self.max_ctx_len, "index is full"
+        hip.require(tuple(k.shape) == want, f"keys shape {tuple(k.shape)} != {want}")        # lib.rs:353
+        hip.require(tuple(v.shape) == want, f"vals shape {tuple(v.shape)} != {want}")        # lib.rs:354
+        hip.require(self.ctx_len < self.max_ctx_len, "index is full")
         hip.append_kv(self.keys, self.vals, k, v, self.ctx_len)
         if self.sketch is not None:
             if self.ctx_len == 0:
@@ -186,7 +186,7 @@ class DiffCacheHIP:
         ef = min(ef, self.ctx_len)
         q = _as_bf16(queries, self.device)
         want = (self.bsz, self.kv_head_num, self.head_dim)
-        assert tuple(q.shape) == want, f"queries shape {tuple(q.shape)} != {want}"     # lib.rs:376
+        hip.require(tuple(q.shape) == want, f"queries shape {tuple(q.shape)} != {want}")     # lib.rs:376
         if ef <= 0:
             empty = torch.empty((self.bsz * self.kv_head_num, 0), dtype=torch.int32, device=self.device)
             return (empty, None) if return_scores else empty
@@ -220,9 +220,9 @@ class DiffCacheHIP:
             shape = (self.bsz, self.kv_head_num, ef_eff, self.head_dim)
             ok = torch.empty(shape, dtype=torch.bfloat16, device=self.device)
             ov = torch.empty(shape, dtype=torch.bfloat16, device=self.device)
-        assert ok.shape[0] == self.bsz and ok.shape[1] == self.kv_head_num and ok.shape[2] >= ef_eff \
-            and ok.shape[3] == self.head_dim, "out_keys must be (bsz, kv_heads, >= ef, head_dim)"
-        assert ov.shape == ok.shape, "out_vals must match out_keys"
+        hip.require(ok.shape[0] == self.bsz and ok.shape[1] == self.kv_head_num and ok.shape[2] >= ef_eff
+                    and ok.shape[3] == self.head_dim, "out_keys must be (bsz, kv_heads, >= ef, head_dim)")
+        hip.require(ov.shape == ok.shape, "out_vals must match out_keys")
         hip.gather_rows(self.keys, self.vals, ids, ok, ov, row_offset=0, n_idx=ef_eff)
         if not dev_out:
             for dst, src in ((out_keys, ok), (out_vals, ov)):
@@ -259,7 +259,7 @@ class DiffCacheHIP:
         return self.keys[:, :, :self.ctx_len].float().cpu().numpy()
 
     def update_r_sq(self, r_sq: Sequence[float]) -> None:
-        assert len(r_sq) == self.kv_head_num, "r_sq length must match kv_head_num"     # lib.rs:652
+        hip.require(len(r_sq) == self.kv_head_num, "r_sq length must match kv_head_num")     # lib.rs:652
         self.r_sq = [float(x) for x in r_sq]
 
     def save(self, path: str) -> None:
@@ -284,9 +284,9 @@ class DiffCacheHIP:
         for b in range(self.bsz):
             for h in range(self.kv_head_num):
                 snap = snapshot.read(f"{path}b{b:03d}_h{h:03d}.idx")
-                assert snap["dim"] == self.head_dim, "snapshot dimension does not match"
+                hip.require(snap["dim"] == self.head_dim, "snapshot dimension does not match")
                 n = snap["n_nodes_stored"]
-                assert n <= self.max_ctx_len, "snapshot longer than max_ctx_len"
+                hip.require(n <= self.max_ctx_len, "snapshot longer than max_ctx_len")
                 n_min = n if n_min is None else min(n_min, n)
                 self.keys[b, h, :n].copy_(torch.from_numpy(snap["keys"]).to(torch.bfloat16))
                 self.vals[b, h, :n].copy_(torch.from_numpy(snap["vals"]).to(torch.bfloat16))

@@ -164,7 +164,7 @@ class DiffCache:
         """key_states / value_states (bsz, seq_len, num_kv_heads, head_dim) bf16 on the
         GPU (diffcache.py:149-184)."""
         seq_len = key_states.size(1)
-        assert seq_len <= self.max_length, "prompt longer than max_length"
+        hip.require(seq_len <= self.max_length, "prompt longer than max_length")
 
         # r_sq from the prefill keys, as the reference does; only the graph build needed it
         r_sq = torch.einsum("bshd,bshd->bsh", key_states, key_states).max(dim=1).values.max(dim=0).values.tolist()
@@ -235,7 +235,8 @@ class DiffCache:
                                  hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
                 self._hook_ws_ready = False   # the one-shot call does not leave the state initialised
             self._ws_ready = False
-        assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
+        hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,
+                    "the recent window is full (kvbuf_suffix_maxlen)")       # diffcache.py:221
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1
 
@@ -261,10 +262,11 @@ class DiffCache:
         (bsz, 1, Hkv, hd).  Returns (bsz, Hq, hd) bf16.  Call it for every layer of
         a step; the suffix grows by one after the last layer."""
         b, hq, hkv, hd = self.batch_size, self.num_q_heads, self.num_kv_heads, self.head_dim
-        assert self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen
+        hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,
+                    "the recent window is full (kvbuf_suffix_maxlen)")       # diffcache.py:221
         lo, hi = self._region()
         pos = hi + self.kvbuf_suffix_len
-        assert pos < self.max_length, "store is full"
+        hip.require(pos < self.max_length, "store is full")
         q = queries.reshape(b, hq, hd)
         if not q.is_contiguous():
             q = q.contiguous()

@@ -60,8 +60,10 @@ class PQIndex:
     def __init__(self, store_k: torch.Tensor, books: torch.Tensor, codes: torch.Tensor,
                  n_cand: int = 4096, topk: int = 1024) -> None:
         b, h, n, hd = store_k.shape
-        assert books.shape[0] == h and books.shape[2] == 256 and books.dtype == torch.float32
-        assert codes.shape == (b * h, n, books.shape[1]) and codes.dtype == torch.uint8
+        hip.require(books.shape[0] == h and books.shape[2] == 256 and books.dtype == torch.float32,
+                    "books must be (kv_heads, M, 256, hd / M) fp32")
+        hip.require(codes.shape == (b * h, n, books.shape[1]) and codes.dtype == torch.uint8,
+                    "codes must be (bsz * kv_heads, n, M) uint8")
         self.store_k, self.books, self.codes = store_k, books.contiguous(), codes.contiguous()
         self.b, self.h, self.n, self.hd, self.m = b, h, n, hd, books.shape[1]
         self.n_cand, self.topk = min(n_cand, n), min(topk, n)

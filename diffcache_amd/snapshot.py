@@ -64,7 +64,8 @@ def write(path: str, keys_f32: np.ndarray, vals_f32: np.ndarray, *, m: int, ef_c
     keys = np.ascontiguousarray(keys_f32, dtype="<f4")
     vals = np.ascontiguousarray(vals_f32, dtype="<f4")
     n, dim = keys.shape
-    assert vals.shape == (n, dim)
+    if vals.shape != (n, dim):
+        raise AssertionError("keys and vals must have the same shape")
     name_b = name.encode("utf-8")
     with open(path, "wb") as f:
         f.write(_nodes_without_edges(n))
