@@ -346,6 +346,11 @@ def gather_rows(store_k: Optional[torch.Tensor], store_v: Optional[torch.Tensor]
     dst = out_k if out_k is not None else out_v
     db, dh, dr = _store_strides(dst)
     n_idx = idx.shape[1] if n_idx is None else n_idx
+    require(idx.dim() == 2 and idx.shape[0] == b * h and idx.shape[1] >= n_idx and idx.element_size() == 4,
+            "idx must be a 32-bit (bsz * kv_heads, >= n_idx) tensor")
+    for o in (out_k, out_v):
+        require(o is None or (o.shape[0] == b and o.shape[1] == h and o.shape[2] >= n_idx and o.shape[3] == hd),
+                "out_k / out_v must be (bsz, kv_heads, >= n_idx, head_dim)")
     _check(lib.dc_gather_rows_bf16(_opt(store_k, "store_k"), _opt(store_v, "store_v"), _dev(idx, "idx"),
                                    _opt(out_k, "out_k"), _opt(out_v, "out_v"), b, h, n_idx,
                                    idx.stride(0), hd, row_offset, sb, sh, sr, db, dh, dr, _stream()))
