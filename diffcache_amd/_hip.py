@@ -468,6 +468,12 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
     if not q.is_contiguous():
         raise DiffCacheError("q must be contiguous")
     group = q.numel() // (b * h * hd)
+    if group < 1 or q.numel() != b * h * group * hd:
+        raise DiffCacheError("q must hold (b, h * group, hd) values")
+    if out.numel() < q.numel() or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise DiffCacheError("out must be a contiguous bf16 tensor of the size of q")
+    if idx_out.dim() != 2 or idx_out.shape[0] < b * h or idx_out.element_size() != 4:
+        raise DiffCacheError("idx_out must be a 32-bit (b * h, >= budget) tensor")
     a = LayerArgs()
     a.q, a.k, a.v = _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v")
     a.new_k, a.new_v = _opt(new_k, "new_k"), _opt(new_v, "new_v")
