@@ -40,6 +40,7 @@ constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
+constexpr int kSharedPollUnits = 16;  // sketch scan: up to this many units, one wave per block polls
 constexpr int kPqThreads = 512;    // PQ scan: threads per block = keys per step
 constexpr int kPqBigSteps = 8;     // PQ scan: 4096 keys per large block
 constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
@@ -281,8 +282,8 @@ __device__ __forceinline__ float sketch_dot16(const uint4 &c, const float (&w)[1
 // yields the bucket of A_k exactly as in score_prune_kernel, and a row is kept when
 // bucket(approx_i + margin) is not worse than the running threshold bucket,
 // margin = 2E' + Q.  The kept rows are rescored exactly by rescore_kernel.
-template <int HD>
-__global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
+template <int HD, bool SHARED_POLL>
+__global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kernel(
     const uint8_t *__restrict__ C, const uint16_t *__restrict__ Q, const float *__restrict__ scale,
     const float *__restrict__ resid, uint32_t *__restrict__ hist, UnitState *__restrict__ state,
     uint2 *__restrict__ surv, int n_units, int n_h, int n_rows, int64_t cb, int64_t ch, int64_t cr,
@@ -290,6 +291,7 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
     constexpr int LPR = HD / 16;  // lanes per row, 16 code bytes each
     __shared__ uint32_t lhist[DC_HIST_BINS];
     __shared__ uint2 stage[kStage];
+    __shared__ uint32_t s_tb;  // the block's copy of the unit's running threshold bucket
     __shared__ uint32_t wtot[kThreads / 64 + 1];
     __shared__ uint32_t s_wcnt[kThreads / 64];
     __shared__ uint32_t s_base;
@@ -352,6 +354,7 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
         margin = dc_sketch_margin(e, wabs, mode);
     }
     if (chunk == 0 && tid == 0) st->margin = __float_as_uint(margin);
+    if (tid == 0) s_tb = tb;
     __syncthreads();
 
     uint2 *wstage = stage + wave * (kBigSteps * 64);
@@ -405,15 +408,31 @@ __global__ __launch_bounds__(kThreads) void sketch_prune_kernel(
     // The threshold poll is issued before the prefetch: loads return in order, so waiting
     // for a poll that was issued last would also wait for the whole prefetch.
     int step = 0;
+    // With few units the whole chip polls a handful of lines, and every poll holds back
+    // the younger loads of its wave (the poll is an agent-scope load): then only wave 0
+    // polls and passes the value on through LDS.  With many units every wave polls for
+    // itself, which keeps its threshold one step fresher.
+    // (SHARED_POLL is a template parameter: as a run-time choice it costs registers.)
     for (; step + 1 < my_steps; step += 2) {
-        uint32_t tb_next = load_relaxed(&st->tb_run);
+        uint32_t tb_next = tb;
+        if (!SHARED_POLL || wave == 0) tb_next = load_relaxed(&st->tb_run);
         load_step(step + 1, cb2);
         work_step(step, ca);
-        tb = tb_next;
-        tb_next = load_relaxed(&st->tb_run);
+        if (SHARED_POLL) {
+            if (wave == 0 && lane == 0) lds_store_relaxed(&s_tb, tb_next);
+            tb = lds_load_relaxed(&s_tb);
+        } else {
+            tb = tb_next;
+        }
+        if (!SHARED_POLL || wave == 0) tb_next = load_relaxed(&st->tb_run);
         load_step(step + 2, ca);
         work_step(step + 1, cb2);
-        tb = tb_next;
+        if (SHARED_POLL) {
+            if (wave == 0 && lane == 0) lds_store_relaxed(&s_tb, tb_next);
+            tb = lds_load_relaxed(&s_tb);
+        } else {
+            tb = tb_next;
+        }
     }
     if (step < my_steps) work_step(step, ca);  // an odd last step; its rows are already on the way
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
@@ -1144,13 +1163,17 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
         if (rc) return rc;
     }
     if (ev_scan_begin) (void)hipEventRecord((hipEvent_t)ev_scan_begin, st);
-#define DC_LAUNCH_SK(HD)                                                                            \
-    hipLaunchKernelGGL(sketch_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st, codes, \
-                       (const uint16_t *)q, scale, resid, w.hist, w.state, w.surv, p.n_units, n_h,       \
-                       n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps)
-    if (hd == 64) DC_LAUNCH_SK(64);
-    else if (hd == 128) DC_LAUNCH_SK(128);
-    else DC_LAUNCH_SK(256);
+#define DC_LAUNCH_SK(HD, SP)                                                                        \
+    hipLaunchKernelGGL((sketch_prune_kernel<HD, SP>), dim3((unsigned)p.blocks), dim3(kThreads), 0, st,  \
+                       codes, (const uint16_t *)q, scale, resid, w.hist, w.state, w.surv, p.n_units,    \
+                       n_h, n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps)
+    const bool shared_poll = p.n_units <= kSharedPollUnits;
+    if (hd == 64 && shared_poll) DC_LAUNCH_SK(64, true);
+    else if (hd == 64) DC_LAUNCH_SK(64, false);
+    else if (hd == 128 && shared_poll) DC_LAUNCH_SK(128, true);
+    else if (hd == 128) DC_LAUNCH_SK(128, false);
+    else if (shared_poll) DC_LAUNCH_SK(256, true);
+    else DC_LAUNCH_SK(256, false);
 #undef DC_LAUNCH_SK
     DC_CHECK_LAUNCH(who);
     if (ev_scan_end) (void)hipEventRecord((hipEvent_t)ev_scan_end, st);
