@@ -40,7 +40,7 @@ constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
-constexpr int kSharedPollUnits = 16;  // sketch scan: up to this many units, one wave per block polls
+constexpr int kSharedPollUnits = 8;   // sketch scan: up to this many units, one wave per block polls
 constexpr int kPqThreads = 512;    // PQ scan: threads per block = keys per step
 constexpr int kPqBigSteps = 8;     // PQ scan: 4096 keys per large block
 constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
