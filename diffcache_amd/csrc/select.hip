@@ -212,27 +212,75 @@ __global__ __launch_bounds__(kFinalThreads) void sort_kernel(
         }
         buf[i] = v;
     }
-    __syncthreads();
-    // Pairs t in [64w, 64w + 64) (and the same range shifted by multiples of the block
-    // size) belong to wave w.  With a stride of at most 64 they lie inside the wave's own
-    // 128 elements, and a wave's LDS operations complete in order, so those stages need no
-    // block barrier: only the stages that cross waves, and the step into one, have one.
-    for (int size = 2; size <= pow2; size <<= 1) {
-        for (int stride = size >> 1, ls = __ffs(size) - 2; stride > 0; stride >>= 1, --ls) {
-            for (int t = tid; t < (pow2 >> 1); t += kFinalThreads) {
-                const int i = ((t >> ls) << (ls + 1)) | (t & (stride - 1));
-                const int j = i + stride;
-                const bool asc = (i & size) == 0;
-                unsigned long long a = buf[i], b = buf[j];
-                if ((a > b) == asc) {
-                    buf[i] = b;
-                    buf[j] = a;
+    if (IN_LDS) {
+        // The list is padded to at least 128 elements, one block of a wave (the padding
+        // sorts to the end).  Stages with a stride of at most 64 stay inside such a block:
+        // the wave keeps the block in registers, two elements per lane, exchanges across
+        // lanes with shuffles and touches LDS once per run of those stages.  Only the
+        // stages that cross waves (stride >= 128) go through LDS with a block barrier.
+        const int n = pow2 < 128 ? 128 : pow2;
+        for (int i = pow2 + tid; i < n; i += kFinalThreads) buf[i] = ~0ull;
+        __syncthreads();
+        const int lane = tid & 63;
+        auto local_stages = [&](int size_lo, int size_hi) {
+            for (int blk = tid >> 6; blk * 128 < n; blk += kFinalThreads / 64) {  // wave-uniform
+                const int i0 = blk * 128 + lane, i1 = i0 + 64;
+                unsigned long long a = buf[i0], b = buf[i1];
+                for (int size = size_lo; size <= size_hi; size <<= 1) {
+                    int s = size >> 1;
+                    if (s >= 64) {  // the two elements of the lane meet; both sort the same way
+                        const bool asc = (i0 & size) == 0;
+                        const unsigned long long lo = a < b ? a : b, hi = a < b ? b : a;
+                        a = asc ? lo : hi;
+                        b = asc ? hi : lo;
+                        s = 32;
+                    }
+                    const bool asc_a = (i0 & size) == 0, asc_b = (i1 & size) == 0;
+                    for (; s >= 1; s >>= 1) {
+                        const unsigned long long pa = __shfl_xor(a, s, 64), pb = __shfl_xor(b, s, 64);
+                        const bool lower = (lane & s) == 0;
+                        a = ((lower == asc_a) == (a < pa)) ? a : pa;  // keep the smaller iff lower == asc
+                        b = ((lower == asc_b) == (b < pb)) ? b : pb;
+                    }
                 }
+                buf[i0] = a;
+                buf[i1] = b;
             }
-            if (!IN_LDS || stride > 64 || (stride == 1 && size >= 128)) __syncthreads();
-            else {
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // compiler ordering only
-                __builtin_amdgcn_wave_barrier();
+        };
+        local_stages(2, 128);
+        __syncthreads();
+        for (int size = 256; size <= n; size <<= 1) {
+            for (int stride = size >> 1, ls = __ffs(size) - 2; stride >= 128; stride >>= 1, --ls) {
+                for (int t = tid; t < (n >> 1); t += kFinalThreads) {
+                    const int i = ((t >> ls) << (ls + 1)) | (t & (stride - 1));
+                    const int j = i + stride;
+                    const bool asc = (i & size) == 0;
+                    unsigned long long a = buf[i], b = buf[j];
+                    if ((a > b) == asc) {
+                        buf[i] = b;
+                        buf[j] = a;
+                    }
+                }
+                __syncthreads();
+            }
+            local_stages(size, size);
+            __syncthreads();
+        }
+    } else {
+        __syncthreads();
+        for (int size = 2; size <= pow2; size <<= 1) {
+            for (int stride = size >> 1, ls = __ffs(size) - 2; stride > 0; stride >>= 1, --ls) {
+                for (int t = tid; t < (pow2 >> 1); t += kFinalThreads) {
+                    const int i = ((t >> ls) << (ls + 1)) | (t & (stride - 1));
+                    const int j = i + stride;
+                    const bool asc = (i & size) == 0;
+                    unsigned long long a = buf[i], b = buf[j];
+                    if ((a > b) == asc) {
+                        buf[i] = b;
+                        buf[j] = a;
+                    }
+                }
+                __syncthreads();
             }
         }
     }
