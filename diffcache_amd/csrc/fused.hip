@@ -713,20 +713,23 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     UnitState *st = state + unit;
     uint32_t n_s = st->surv_cnt;
     if (n_s > (uint32_t)n_rows) n_s = n_rows;
-    const uint32_t per = ((n_s + (uint32_t)nblk - 1) / (uint32_t)nblk + kPer - 1) / kPer * kPer;
-    const uint32_t lo = (uint32_t)blk * per;
-    uint32_t hi = lo + per;
-    if (hi > n_s) hi = n_s;
-    if (lo >= n_s) return;
+    // The list is dealt to the unit's blocks in tiles of kThreads entries, round robin:
+    // the scan appends in the order its blocks finish, and the entries of late blocks
+    // (tight threshold) pass the filter far more often than those of early ones, so
+    // contiguous slices would leave a few blocks with most of the gathers.
+    const uint32_t n_tiles = (n_s + kThreads - 1) / kThreads;
+    if ((uint32_t)blk >= n_tiles) return;
+    const uint32_t my_tiles = (n_tiles - (uint32_t)blk + (uint32_t)nblk - 1) / (uint32_t)nblk;
+    auto entry = [&](uint32_t t) { return ((uint32_t)blk + t * (uint32_t)nblk) * kThreads + (uint32_t)tid; };
 
     // the block's first batch of the list is requested before the threshold is worked out
     const uint2 *su = surv + (int64_t)unit * n_rows;
     uint2 p[kRescoreBatch];
 #pragma unroll
     for (int j = 0; j < kRescoreBatch; ++j) {
-        const uint32_t i = lo + j * kThreads + tid;
+        const uint32_t i = entry((uint32_t)j);
         p[j] = make_uint2(0u, 0u);
-        if (i < hi) p[j] = su[i];
+        if ((uint32_t)j < my_tiles && i < n_s) p[j] = su[i];
     }
     uint32_t tb, c_less;
     unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
@@ -738,16 +741,18 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     uint32_t *ck = cand_key + (int64_t)unit * n_rows;
     uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
 
-    for (uint32_t i0 = lo; i0 < hi; i0 += kPer) {
+    for (uint32_t t0 = 0; t0 < my_tiles; t0 += kRescoreBatch) {
         uint32_t pass = 0;
 #pragma unroll
         for (int j = 0; j < kRescoreBatch; ++j) {
-            const uint32_t i = i0 + j * kThreads + tid;
-            if (i0 != lo) {
+            const uint32_t t = t0 + (uint32_t)j;
+            const uint32_t i = entry(t);
+            const bool in = t < my_tiles && i < n_s;
+            if (t0 != 0) {
                 p[j] = make_uint2(0u, 0u);
-                if (i < hi) p[j] = su[i];
+                if (in) p[j] = su[i];
             }
-            if (i < hi && dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
+            if (in && dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
         }
         uint32_t n_c;
         uint32_t pos = block_excl_scan<kThreads>(__popc(pass), wtot, &n_c);
