@@ -397,7 +397,9 @@ def kcheck(scores: torch.Tensor, n_sel: int, hd: int, k_check_seq, attn_mass_thr
     if scores.dtype != torch.float32 or scores.dim() != 2 or scores.stride(1) != 1:
         raise DiffCacheError("scores must be a 2-d fp32 tensor with contiguous rows")
     n_units = scores.shape[0]
-    seq = [int(x) for x in k_check_seq][:16]
+    seq = [int(x) for x in k_check_seq]
+    if len(seq) > 16:
+        raise DiffCacheError(f"k_check_seq holds {len(seq)} sizes; dc_kcheck_f32 takes at most 16")
     arr = (C.c_int * max(len(seq), 1))(*seq)
     if n_eff is None:
         n_eff = torch.empty((n_units,), dtype=torch.int32, device=scores.device)

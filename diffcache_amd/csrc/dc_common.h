@@ -78,7 +78,7 @@ __device__ __forceinline__ uint32_t dc_f2ord(float x) {
 }
 
 // Histogram bucket of a score (larger score = better = smaller bucket), a monotone
-// map onto [0, DC_HIST_BINS).  Positive scores from 2^-20 up to 2^20 get 32 buckets
+// map onto [0, DC_HIST_BINS).  Positive scores from 2^-20 up to 2^20 get 8 buckets
 // per binade (the top-k of an attention scan lives there: a finer grid leaves
 // fewer rows in the threshold bucket, a coarser one costs the scan fewer histogram
 // atomics); smaller positives share the last fine bucket, larger ones the first;

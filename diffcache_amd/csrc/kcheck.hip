@@ -14,6 +14,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kMaxSeq = 16;
 constexpr int kMinRank = 5;  // nsw.rs:288
+constexpr int kMaxEf = 16384;  // nsw.rs:15: sizes beyond the reference's ln(rank) table never pass (nsw.rs:207-210)
 
 struct KSeq {
     int h[kMaxSeq];
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void kcheck_kernel(const float *__restric
     for (int e = 0; e < seq.n; ++e) {
         const int H = seq.h[e];
         float alpha = nan, mass = nan;
-        if (!decided && H < n_sel && H > kMinRank) {
+        if (!decided && H < n_sel && H > kMinRank && H <= kMaxEf) {
             // least squares of logit against ln(rank) over ranks kMinRank..H
             double sx = 0.0, sy = 0.0, sxx = 0.0, sxy = 0.0;
             for (int i = kMinRank - 1 + tid; i < H; i += kThreads) {

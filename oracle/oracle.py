@@ -479,6 +479,7 @@ def pq_search(q_u16: np.ndarray, k_u16: np.ndarray, codes: np.ndarray, lut_f32: 
 # --------------------------------------------------------------------------
 
 K_CHECK_MIN_RANK = 5  # nsw.rs:288
+MAX_EF = 16384        # nsw.rs:15: length of the reference's ln(rank) table
 
 
 def fit_alpha_from_logits(logits_sorted: np.ndarray, min_rank: int) -> Optional[np.float32]:
@@ -487,6 +488,8 @@ def fit_alpha_from_logits(logits_sorted: np.ndarray, min_rank: int) -> Optional[
     z = np.asarray(logits_sorted, dtype=np.float32)
     h = len(z)
     if h == 0 or min_rank == 0 or min_rank >= h:
+        return None
+    if h > MAX_EF:      # the reference's ln(rank) table ends there (nsw.rs:15,207-210)
         return None
     n = float(h - min_rank + 1)
     if n < 2.0:
@@ -570,7 +573,7 @@ def k_check_budget(dists_sorted: np.ndarray, dim: int, k_check_seq: Sequence[int
 
 def coarse_bucket(scores: np.ndarray, mode: int) -> np.ndarray:
     """Bucket (smaller = better) of each score: positive scores in [2^-20, 2^20) get
-    32 buckets per binade, clamped outside; negative scores two per binade."""
+    8 buckets per binade, clamped outside; negative scores two per binade."""
     s = np.asarray(scores, dtype=np.float32)
     if mode == MODE_REF_DIST:
         d = ref_dist(s)

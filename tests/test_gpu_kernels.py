@@ -648,6 +648,25 @@ def test_kcheck_matches_oracle(mode):
     kcheck_case(scores[:, :150], 64, [3, 5, 6, 100, 150, 200], 0.7, mode)   # sizes <= 5 and >= n_sel
 
 
+def test_kcheck_sizes_beyond_the_reference_table_never_pass():
+    """nsw.rs:15,207-210: fit_alpha_from_logits returns None when H > MAX_EF = 16384, so with
+    ef = 20000 a size of 16385 or more is never accepted, however steep the power law."""
+    hd, n_sel = 128, 20000
+    sq = np.sqrt(np.float32(hd))
+    r = np.arange(1, n_sel + 1, dtype=np.float64)
+    rows = [np.sort(((12.0 - a * np.log(r)) * sq).astype(np.float32))[::-1] for a in (3.0, 2.0)]
+    scores = np.ascontiguousarray(np.stack(rows))
+    for mode in (0, 1):
+        kcheck_case(scores, hd, [16385, 18000, 19999], 0.5, mode)
+        n_eff = hip.kcheck(torch.from_numpy(scores).to(DEV), n_sel, hd, [16385, 18000], 0.5, mode)
+        assert n_eff.tolist() == [n_sel, n_sel]
+        kcheck_case(scores, hd, [16384, 18000], 0.5, mode)
+        n_eff = hip.kcheck(torch.from_numpy(scores).to(DEV), n_sel, hd, [16384, 18000], 0.5, mode)
+        assert n_eff.tolist() == [16384, 16384]
+    with pytest.raises(hip.DiffCacheError):
+        hip.kcheck(torch.from_numpy(scores).to(DEV), n_sel, hd, list(range(100, 1800, 100)), 0.5)
+
+
 def test_kcheck_and_sketch_edge_sizes():
     # no sizes to check -> the whole list; an empty list -> 0
     sc = torch.sort(torch.randn((3, 40), device=DEV), dim=1, descending=True).values.contiguous()

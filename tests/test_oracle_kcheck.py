@@ -36,6 +36,22 @@ def test_fit_alpha_guards():
     assert orc.fit_alpha_from_logits(z[:5], 5) is None                         # min_rank >= h
     assert orc.fit_alpha_from_logits(z[:6], 5) is not None                     # n == 2 is enough
     assert float(orc.fit_alpha_from_logits(z, 5)) == 0.0                       # flat logits
+    # nsw.rs:15,207-210: the ln(rank) table holds MAX_EF = 16384 entries; a longer list is never fitted
+    r = np.arange(1, 16386, dtype=np.float64)
+    zl = (10.0 - 2.0 * np.log(r)).astype(np.float32)
+    assert orc.MAX_EF == 16384
+    assert abs(float(orc.fit_alpha_from_logits(zl[:16384], 5)) - 2.0) < 1e-4
+    assert orc.fit_alpha_from_logits(zl[:16385], 5) is None
+
+
+def test_budget_never_stops_at_a_size_beyond_max_ef():
+    # a steep power law passes at every size up to 16384 and can never pass beyond it
+    sq = np.sqrt(np.float32(128))
+    r = np.arange(1, 20001, dtype=np.float64)
+    s = ((12.0 - 3.0 * np.log(r)) * sq).astype(np.float32)
+    d = orc.ref_dist(s)
+    assert orc.k_check_budget(d, 128, [16384, 18000], 0.5) == 16384
+    assert orc.k_check_budget(d, 128, [16385, 18000], 0.5) == 20000
 
 
 def test_mass_hand_values():
