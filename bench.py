@@ -145,16 +145,27 @@ def cpu_baseline(torch, cfg, layers_data, target_s: float = 10.0):
     }
 
 
-def run_pq(args, torch, hip, dev) -> int:
-    """Benchmark configuration 4: PQ baseline, one layer, 8 kv heads x 1,048,576 keys, M 32 x 8-bit
-    codes, ADC scan -> 4096 candidates -> exact bf16 rerank to top-k 1024."""
+def make_pq_index(torch, hip, dev, store=None):
+    """Benchmark configuration 4: 8 kv heads x 1,048,576 keys ~ N(0,1), hd 128, M 32 x 256 centroids
+    from seeded k-means on a 65,536-key sample, 8-bit codes, 4096 candidates, top-k 1024.
+    Returns (index, key store, queries).  `store`: a (1, 8, 2^20, 128) bf16 buffer to fill."""
     from diffcache_amd.pq import PQIndex
     h, n, hd, m, n_cand, topk = 8, 1 << 20, 128, 32, 4096, 1024
     g = torch.Generator(device=dev).manual_seed(4000)
-    t_gen = time.perf_counter()
-    store = torch.empty((1, h, n, hd), dtype=torch.bfloat16, device=dev).normal_(generator=g)
+    if store is None:
+        store = torch.empty((1, h, n, hd), dtype=torch.bfloat16, device=dev)
+    store.normal_(generator=g)
     q = torch.randn((h, hd), generator=g, device=dev).to(torch.bfloat16)
     index = PQIndex.build(store, m=m, sample=65536, iters=8, seed=4000, n_cand=n_cand, topk=topk)
+    return index, store, q
+
+
+def run_pq(args, torch, hip, dev) -> int:
+    """Benchmark configuration 4: PQ baseline, one layer, 8 kv heads x 1,048,576 keys, M 32 x 8-bit
+    codes, ADC scan -> 4096 candidates -> exact bf16 rerank to top-k 1024."""
+    h, n, hd, m, n_cand, topk = 8, 1 << 20, 128, 32, 4096, 1024
+    t_gen = time.perf_counter()
+    index, store, q = make_pq_index(torch, hip, dev)
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t_gen
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps)]

@@ -1,0 +1,186 @@
+"""GPU parity at the launch shapes bench.py times, on bench.py's own data laws.
+
+Every test builds one layer with ``bench.make_layer`` (same seeds, same laws as the timed
+run), drives the call path the benchmark drives (``dc_decode_layer`` with the 8-bit
+sketch, ORDER_ANY, REF_DIST keys, the select state left ready by the previous call) and
+checks it against the CPU oracle:
+
+  config 3  64 units x 131004 rows, k 2048  (one full layer of the 32-layer step)
+  config 2  8 units x 32700 rows, k 1024
+  config 5  8 units x 1048508 rows, k 4096
+  config 4  8 units x 1048576 PQ codes, 4096 candidates -> top 1024
+
+Bars: ids bit-exact against ``oracle.topk_select`` of the GPU's own dense fp32 scores
+(search_bruteforce's kept set, diffcache_cpu/src/nsw.rs:592-630); scores within 1e-5
+relative of a float64 dot; attention within 2e-3 absolute of a float64 softmax
+(src/diffcache/base.py:134-142).  The worst errors against those literal bars are printed.
+"""
+import numpy as np
+import pytest
+import torch
+
+import bench
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+hip = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global hip
+    from diffcache_amd import _hip
+    hip = _hip
+    yield
+    torch.cuda.empty_cache()
+
+
+def u16(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def build_layer(cfg_name: str, cfg_id: int, layer: int = 0):
+    cfg = bench.CONFIGS[cfg_name]
+    b, hkv, n, hd = cfg["batch"], cfg["hkv"], cfg["ctx"], cfg["hd"]
+    dev = torch.device(DEV)
+    v = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    k = torch.empty((b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
+    k, v, q, nk, nv = bench.make_layer(torch, cfg, layer, cfg_id, dev, k, v)
+    return cfg, k, v, q, nk, nv
+
+
+def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units):
+    """The benchmark's layer call on its three routes against the oracle."""
+    cfg, k, v, q, nk, nv = build_layer(cfg_name, cfg_id)
+    b, hq, hkv, hd, n = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["hd"], cfg["ctx"]
+    sink, recent, budget = cfg["sink"], cfg["recent"], cfg["budget"]
+    grp, n_units = hq // hkv, b * hkv
+    lo, hi = sink, n - recent
+    region = hi - lo
+    k_eff = min(budget, region)
+    attended = k_eff + sink + recent + 1
+    mode = hip.MODE_REF_DIST
+    print(f"{cfg_name}: {n_units} units x {region} rows, k {k_eff}", flush=True)
+
+    sketch = hip.Sketch(k).build(k, lo, region)
+    ws = hip.alloc_workspace(hip.layer_workspace_bytes(n_units, region, budget, grp, hd, attended), DEV)
+    idx = {r: torch.full((n_units, budget), -1, dtype=torch.int32, device=DEV) for r in ("sketch", "stream", "dense")}
+    out = {r: torch.empty((b, hq, hd), dtype=torch.bfloat16, device=DEV) for r in idx}
+    scores = torch.empty((n_units, region), dtype=torch.float32, device=DEV)
+
+    # the default route, as bench.py calls it: twice, the second call on the state the first left
+    for rep in range(2):
+        hip.decode_layer(q, k, v, sink, hi, recent, budget, None, idx["sketch"], out["sketch"], ws, nk, nv,
+                         mode=mode, order=hip.ORDER_ANY, select_state_ready=rep > 0, sketch=sketch)
+    # --scan bf16: the streaming select over the bf16 keys, on the state the sketch route left
+    hip.decode_layer(q, k, v, sink, hi, recent, budget, None, idx["stream"], out["stream"], ws, nk, nv,
+                     mode=mode, order=hip.ORDER_ANY, select_state_ready=True)
+    # --dense: fp32 scores + dc_topk_select
+    hip.decode_layer(q, k, v, sink, hi, recent, budget, scores, idx["dense"], out["dense"], ws, nk, nv,
+                     mode=mode, order=hip.ORDER_ANY)
+    torch.cuda.synchronize()
+
+    sc = scores.cpu().numpy()
+    ids = {r: np.sort(t.cpu().numpy()[:, :k_eff].astype(np.int64), axis=1) for r, t in idx.items()}
+    for u in range(n_units):
+        want = np.sort(orc.topk_select(sc[u], k_eff, orc.MODE_REF_DIST).astype(np.int64))
+        for r in ids:
+            assert np.array_equal(ids[r][u], want), (cfg_name, r, u)
+    del scores
+
+    # scores of a few units against a float64 dot: the bar of the tests (1e-5 of sum |q_i k_i|)
+    # and the literal one (1e-5 of |s|, where |s| is not tiny)
+    qmean = orc.group_mean_bf16(u16(q), hkv)                      # (b, hkv, hd)
+    worst_bar, worst_lit = 0.0, 0.0
+    for u in score_units:
+        bi, h = divmod(u, hkv)
+        rows = u16(k[bi, h, lo:hi])
+        want = orc.scores_f64(qmean[bi, h], rows)
+        err = np.abs(sc[u] - want)
+        bound = 1e-5 * (np.abs(orc.bf16_to_f32(rows).astype(np.float64))
+                        @ np.abs(orc.bf16_to_f32(qmean[bi, h]).astype(np.float64)))
+        assert np.all(err <= bound + 1e-30), (cfg_name, "scores", u)
+        worst_bar = max(worst_bar, float(np.max(err / (bound + 1e-30))))
+        big = np.abs(want) >= 1.0
+        worst_lit = max(worst_lit, float(np.max(err[big] / np.abs(want[big]))))
+    print(f"{cfg_name}: worst score error = {worst_bar:.3f} of the 1e-5*sum|q_i k_i| bar; "
+          f"{worst_lit:.2e} relative to |s| (literal bar 1e-5, rows with |s| >= 1)", flush=True)
+
+    # attention of a few units against the float64 softmax over the oracle's row set
+    worst_abs, worst_small, worst_ulp = 0.0, 0.0, 0.0
+    got = {r: orc.bf16_to_f32(u16(t)) for r, t in out.items()}
+    for u in attn_units:
+        bi, h = divmod(u, hkv)
+        sel = orc.topk_select(sc[u], k_eff, orc.MODE_REF_DIST).astype(np.int64) + lo
+        rows = np.concatenate([sel, np.arange(sink), np.arange(hi, hi + recent)])
+        rows_t = torch.from_numpy(rows).to(DEV)
+        want, _ = orc.sparse_attention(u16(q[bi, h * grp:(h + 1) * grp]), u16(k[bi, h][rows_t]),
+                                       u16(v[bi, h][rows_t]), u16(nk[bi, h]), u16(nv[bi, h]))
+        for r in got:
+            g = got[r][bi, h * grp:(h + 1) * grp]
+            tol = np.maximum(2e-3, np.abs(want) * 2.0 ** -8)
+            assert np.all(np.abs(g - want) <= tol), (cfg_name, "attention", r, u)
+            err = np.abs(g - want)
+            worst_abs = max(worst_abs, float(err.max()))
+            small = np.abs(want) < 0.5          # where bf16 can represent a 2e-3 step at all
+            worst_small = max(worst_small, float(err[small].max()) if small.any() else 0.0)
+            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 1e-30))) - 7)
+            worst_ulp = max(worst_ulp, float((err / ulp).max()))
+    print(f"{cfg_name}: worst attention error = {worst_abs:.2e} absolute; {worst_small:.2e} where |out| < 0.5 "
+          f"(literal bar 2e-3); {worst_ulp:.2f} bf16 ulps of the output (0.5 = correctly rounded)", flush=True)
+    return ids["dense"], sc
+
+
+def test_config3_one_full_layer_all_routes():
+    """64 units: the scan runs as sketch_prune_kernel<128, per-wave poll>, the instantiation the
+    headline figure times; clustered queries (0.7 cluster mean + 0.3 noise)."""
+    check_layer("c3", 3, attn_units=[0, 9, 31, 46, 63], score_units=[0, 21, 63])
+
+
+def test_config2_layer_all_routes():
+    check_layer("c2", 2, attn_units=list(range(8)), score_units=list(range(8)))
+
+
+def test_config5_layer_all_routes():
+    """8 units x 2^20 rows in 256 tight clusters, k 4096: the ids of all routes equal the
+    oracle's, and the size-independent invariants of an exact top-k hold."""
+    ids, sc = check_layer("c5", 5, attn_units=[0, 3, 7], score_units=[0, 5])
+    key = orc.key32(sc.reshape(-1), orc.MODE_REF_DIST).reshape(sc.shape).astype(np.int64)
+    for u in range(ids.shape[0]):
+        chosen = np.zeros(sc.shape[1], bool)
+        chosen[ids[u]] = True
+        assert chosen.sum() == ids.shape[1]                              # no duplicates
+        worst_in, best_out = key[u][chosen].max(), key[u][~chosen].min()
+        assert worst_in <= best_out                                      # every kept key <= every dropped key
+        if worst_in == best_out:                                         # ties at the boundary: lower ids kept
+            tie_in = np.flatnonzero(chosen & (key[u] == worst_in))
+            tie_out = np.flatnonzero(~chosen & (key[u] == worst_in))
+            assert tie_in.max() < tie_out.min()
+
+
+def test_config4_pq_search_full_size():
+    """8 x 2^20 keys, trained codebooks (bench.py's index): the candidate set of dc_pq_search_bf16
+    is the oracle's top-4096 of the GPU's ADC scores, and the final ids are the oracle's top-1024
+    of the candidates' exact scores, best first."""
+    index, store, q = bench.make_pq_index(torch, hip, torch.device(DEV))
+    n_units, n_cand, topk = index.b * index.h, index.n_cand, index.topk
+    lut = hip.pq_build_lut(q, index.books, index.b)
+    adc = hip.pq_adc_scan(index.codes, lut).cpu().numpy()
+    # topk == n_cand: the call returns every candidate (reranked), i.e. the first stage's set
+    cand = hip.pq_search(store, index.codes, lut, q, n_cand, n_cand).cpu().numpy().astype(np.int64)
+    final = index.search(q).cpu().numpy().astype(np.int64)
+    final2 = index.search(q).cpu().numpy().astype(np.int64)     # on the state the first search left
+    for u in range(n_units):
+        want_c = orc.topk_select(adc[u], n_cand, orc.MODE_IP).astype(np.int64)
+        assert np.array_equal(np.sort(cand[u]), np.sort(want_c)), ("candidates", u)
+        ws = np.sort(want_c)
+        exact = hip.score_gathered(store, q, torch.from_numpy(np.tile(ws, (n_units, 1)).astype(np.int32)).to(DEV))
+        ex = exact[u].cpu().numpy()
+        pos = orc.topk_select(ex, topk, orc.MODE_IP).astype(np.int64)
+        assert np.array_equal(final[u], ws[pos]), ("final", u)
+        assert np.array_equal(final2[u], final[u])
+        # the exact scores themselves: float64 dot of the bf16 values
+        want = orc.scores_f64(u16(q[u]), u16(store[u // index.h, u % index.h][torch.from_numpy(ws).to(DEV)]))
+        assert np.max(np.abs(ex - want)) <= 1e-5 * np.max(np.abs(want)) + 1e-4
