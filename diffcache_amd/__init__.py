@@ -4,7 +4,7 @@
 (src/diffcache/kvcache/diffcache.py), ``DiffCacheHIP`` mirrors its native data
 layer (diffcache_cpu/src/lib.rs ``DiffCacheCPU``); both run on hand-written HIP
 kernels behind the C ABI of ``include/diffcache_hip.h``.  Importing the package
-needs the built ``libdiffcache_hip.so`` (``python -m diffcache_amd.build``).
+needs the built ``libdiffcache_hip.so`` (``python diffcache_amd/build.py``).
 """
 from . import _hip
 from .data_layer import DiffCacheHIP, init_metrics, metrics

@@ -27,7 +27,7 @@ LIB_PATH = os.path.join(_HERE, "libdiffcache_hip.so")
 SYMBOLS = (
     "dc_version", "dc_last_error", "dc_group_mean_bf16", "dc_score_bf16",
     "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
-    "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_append_kv_bf16",
+    "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_gather_attn_static_bf16", "dc_append_kv_bf16",
     "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
@@ -64,7 +64,7 @@ class LayerArgs(C.Structure):
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m diffcache_amd.build` "
+            f"{LIB_PATH} is missing: build it with `python diffcache_amd/build.py` "
             "(hipcc, --offload-arch=gfx950). There is no fallback path.")
     lib = C.CDLL(LIB_PATH)
     i, i64, p, sz, f = C.c_int, C.c_int64, C.c_void_p, C.c_size_t, C.c_float
@@ -79,6 +79,8 @@ def _load() -> C.CDLL:
         "dc_attn_workspace_bytes": (sz, [i, i, i, i]),
         "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i,
                                     i64, i64, i64, i64, i64, i64, f, p, sz, p]),
+        "dc_gather_attn_static_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i,
+                                           i64, i64, i64, i64, i64, i64, f, p]),
         "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, i64, i64, i64, p]),
         "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
         "dc_layer_workspace_bytes": (sz, [i, i, i, i, i, i]),
@@ -385,6 +387,33 @@ def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
         hd, n_idx, 0 if idx is None else idx.stride(0), _opt(n_idx_unit, "n_idx_unit"), region_lo, n_sink,
         recent_lo, n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, _dev(workspace, "workspace"), workspace.numel(),
         _stream()))
+    return out
+
+
+def gather_attn_static(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
+                       idx: Optional[torch.Tensor], n_idx: int, region_lo: int, n_sink: int, recent_lo: int,
+                       n_recent: int, out: torch.Tensor, new_k: Optional[torch.Tensor] = None,
+                       new_v: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                       lse: Optional[torch.Tensor] = None,
+                       n_idx_unit: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gather_attn`` without a workspace and without any allocation (dc_gather_attn_static_bf16):
+    the split partials live in a static device array of the library.  q, new_k, new_v must be
+    contiguous and ``out`` is the caller's; sizes beyond the array raise DiffCacheError."""
+    ksb, ksh, ksr = _store_strides(store_k)
+    vsb, vsh, vsr = _store_strides(store_v)
+    b, h, _, hd = store_k.shape
+    for t, name in ((q, "q"), (new_k, "new_k"), (new_v, "new_v"), (out, "out")):
+        if t is not None and not t.is_contiguous():
+            raise DiffCacheError(f"{name} must be contiguous")
+    group = q.numel() // (b * h * hd)
+    if out.dtype != torch.bfloat16 or out.numel() < q.numel():
+        raise DiffCacheError("out must be a bf16 tensor of the size of q")
+    scale = 1.0 / math.sqrt(hd) if scale is None else scale
+    _check(lib.dc_gather_attn_static_bf16(
+        _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v"), _opt(idx, "idx"),
+        _opt(new_k, "new_k"), _opt(new_v, "new_v"), _dev(out, "out"), _opt(lse, "lse"), b, h, group,
+        hd, n_idx, 0 if idx is None else idx.stride(0), _opt(n_idx_unit, "n_idx_unit"), region_lo, n_sink,
+        recent_lo, n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, _stream()))
     return out
 
 

@@ -1,6 +1,7 @@
 """Builds libdiffcache_hip.so in-tree with hipcc for gfx950.
 
-`python -m diffcache_amd.build` — cross-compiles without a GPU.
+`python diffcache_amd/build.py` (or `make -C diffcache_amd/csrc`) — cross-compiles without a
+GPU.  Run it as a script, not with `-m`: importing the package needs the library this builds.
 """
 import os
 import subprocess

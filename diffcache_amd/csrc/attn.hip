@@ -16,6 +16,7 @@
 // Bound by HBM: 2 * HD*2 bytes per row.
 #include "dc_common.h"
 #include <math.h>
+#include <mutex>
 
 namespace {
 
@@ -340,43 +341,45 @@ extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_
     return carve_attn(nullptr, n_units, group, hd, plan_attn(hd, group, n_rows_attended).n_splits).bytes;
 }
 
-extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
-                                   const void *new_k, const void *new_v, void *out, float *lse,
-                                   int n_b, int n_h, int group, int hd, int n_idx,
-                                   int64_t idx_unit_stride, const uint32_t *n_idx_unit,
-                                   int64_t region_lo, int n_sink,
-                                   int64_t recent_lo, int n_recent, int64_t ksb, int64_t ksh,
-                                   int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
-                                   void *workspace, size_t workspace_bytes, void *stream) {
-    DC_REQUIRE(q && k && v && out, "dc_gather_attn_bf16: null pointer");
+namespace {
+
+// Argument checks and the two launches shared by dc_gather_attn_bf16 (caller's workspace) and
+// dc_gather_attn_static_bf16 (the library's static scratch array).
+int gather_attn_common(const char *who, const void *q, const void *k, const void *v, const uint32_t *idx,
+                       const void *new_k, const void *new_v, void *out, float *lse, int n_b, int n_h,
+                       int group, int hd, int n_idx, int64_t idx_unit_stride, const uint32_t *n_idx_unit,
+                       int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent, int64_t ksb,
+                       int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
+                       void *workspace, size_t workspace_bytes, void *stream) {
+    DC_REQUIRE(q && k && v && out, "%s: null pointer", who);
     DC_REQUIRE(n_b >= 0 && n_h >= 1 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
-               "dc_gather_attn_bf16: bad sizes");
-    DC_REQUIRE(n_idx == 0 || idx, "dc_gather_attn_bf16: idx is null but n_idx > 0");
+               "%s: bad sizes", who);
+    DC_REQUIRE(n_idx == 0 || idx, "%s: idx is null but n_idx > 0", who);
     DC_REQUIRE((new_k == nullptr) == (new_v == nullptr),
-               "dc_gather_attn_bf16: new_k and new_v must both be set or both be null");
-    DC_REQUIRE(group >= 1 && group <= 8, "dc_gather_attn_bf16: group %d not in [1,8]", group);
-    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "dc_gather_attn_bf16: head_dim %d unsupported", hd);
+               "%s: new_k and new_v must both be set or both be null", who);
+    DC_REQUIRE(group >= 1 && group <= 8, "%s: group %d not in [1,8]", who, group);
+    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d unsupported", who, hd);
     DC_REQUIRE(dc_aligned16(k) && dc_aligned16(v) && dc_aligned16(q) &&
                    (!new_k || (dc_aligned16(new_k) && dc_aligned16(new_v))),
-               "dc_gather_attn_bf16: pointers must be 16-byte aligned");
+               "%s: pointers must be 16-byte aligned", who);
     DC_REQUIRE(ksb % 8 == 0 && ksh % 8 == 0 && ksr % 8 == 0 && vsb % 8 == 0 && vsh % 8 == 0 &&
                    vsr % 8 == 0,
-               "dc_gather_attn_bf16: strides must be multiples of 8 elements");
-    DC_REQUIRE(idx_unit_stride >= n_idx, "dc_gather_attn_bf16: idx_unit_stride < n_idx");
+               "%s: strides must be multiples of 8 elements", who);
+    DC_REQUIRE(idx_unit_stride >= n_idx, "%s: idx_unit_stride < n_idx", who);
     DC_REQUIRE(region_lo >= 0 && recent_lo >= 0 && recent_lo + n_recent < 0xffffffffll,
-               "dc_gather_attn_bf16: row numbers out of range");
+               "%s: row numbers out of range", who);
     const int n_units = n_b * n_h;
     if (n_units == 0) return DC_OK;
     const int n_total = n_idx + n_sink + n_recent + (new_k ? 1 : 0);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
-               "dc_gather_attn_bf16: workspace must be non-null and 256-byte aligned");
+               "%s: workspace must be non-null and 256-byte aligned", who);
     const AttnPlan plan = plan_attn(hd, group, n_total);
     const AttnWs w = carve_attn(workspace, n_units, group, hd, plan.n_splits);
     if (workspace_bytes < w.bytes) {
-        dc_set_error("dc_gather_attn_bf16: workspace %zu bytes < %zu needed", workspace_bytes, w.bytes);
+        dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, w.bytes);
         return DC_ENOMEM;
     }
-    DC_REQUIRE((int64_t)n_units * plan.n_splits < (1ll << 31), "dc_gather_attn_bf16: grid too large");
+    DC_REQUIRE((int64_t)n_units * plan.n_splits < (1ll << 31), "%s: grid too large", who);
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)((size_t)n_units * plan.n_splits));
     int rc;
@@ -395,12 +398,87 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
         rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                               plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
-    DC_REQUIRE(rc == 0, "dc_gather_attn_bf16: unsupported group %d", group);
-    DC_CHECK_LAUNCH("dc_gather_attn_bf16(attn)");
+    DC_REQUIRE(rc == 0, "%s: unsupported group %d", who, group);
+    DC_CHECK_LAUNCH(who);
     hipLaunchKernelGGL(merge_kernel, dim3((unsigned)(n_units * group)), dim3(hd), 0, st, w.acc, w.ml, o16,
                        lse, group, hd, plan.n_splits);
-    DC_CHECK_LAUNCH("dc_gather_attn_bf16(merge)");
+    DC_CHECK_LAUNCH(who);
     return DC_OK;
+}
+
+// Scratch of the allocation-free entry point: the per-split (m, l, acc) partials.  One copy
+// per GPU, held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address is looked up once per device and kept.
+constexpr size_t kStaticScratchBytes = (size_t)DC_ATTN_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
+                                   const void *new_k, const void *new_v, void *out, float *lse,
+                                   int n_b, int n_h, int group, int hd, int n_idx,
+                                   int64_t idx_unit_stride, const uint32_t *n_idx_unit,
+                                   int64_t region_lo, int n_sink,
+                                   int64_t recent_lo, int n_recent, int64_t ksb, int64_t ksh,
+                                   int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+    return gather_attn_common("dc_gather_attn_bf16", q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group,
+                              hd, n_idx, idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo,
+                              n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, workspace, workspace_bytes,
+                              stream);
+}
+
+extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
+                                          const void *new_k, const void *new_v, void *out, float *lse,
+                                          int n_b, int n_h, int group, int hd, int n_idx,
+                                          int64_t idx_unit_stride, const uint32_t *n_idx_unit,
+                                          int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
+                                          int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
+                                          int64_t vsr, float scale, void *stream) {
+    const char *who = "dc_gather_attn_static_bf16";
+    DC_REQUIRE(n_b >= 0 && n_h >= 1 && group >= 1 && group <= 8 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
+               "%s: bad sizes", who);
+    DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d unsupported", who, hd);
+    const int64_t n_units = (int64_t)n_b * n_h;
+    DC_REQUIRE(n_units < (1 << 20), "%s: too many units", who);
+    const int64_t n_total = (int64_t)n_idx + n_sink + n_recent + (new_k ? 1 : 0);
+    DC_REQUIRE(n_total < (1ll << 31), "%s: too many rows", who);
+    const size_t need = dc_attn_workspace_bytes((int)n_units, group, hd, (int)n_total);
+    if (need > kStaticScratchBytes) {
+        dc_set_error("%s: %lld units x %lld attended rows (group %d, head_dim %d) need %zu bytes of scratch; "
+                     "the static scratch holds %zu (use dc_gather_attn_bf16 with a workspace)",
+                     who, (long long)n_units, (long long)n_total, group, hd, need, kStaticScratchBytes);
+        return DC_ENOMEM;
+    }
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        dc_set_error("%s: no current device (or device number >= %d)", who, kMaxDevices);
+        return DC_EINVAL;
+    }
+    void *ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ptr = g_scratch_ptr[dev];
+        if (!ptr) {
+            // once per device, with that device current: every GPU has its own copy of the array
+            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr) {
+                dc_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev,
+                             hipGetErrorString(e));
+                return DC_ELAUNCH;
+            }
+            g_scratch_ptr[dev] = ptr;
+        }
+    }
+    // Every split slot the merge reads is written by the attention kernel of the same call, so
+    // nothing has to start at zero; the contents of the previous call are simply overwritten.
+    return gather_attn_common(who, q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group, hd, n_idx,
+                              idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo, n_recent, ksb, ksh,
+                              ksr, vsb, vsh, vsr, scale, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int dc_gather_rows_bf16(const void *k, const void *v, const uint32_t *idx, void *out_k,

@@ -217,6 +217,29 @@ int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint3
                         void *stream);
 
 /*
+ * dc_gather_attn_bf16 for callers that cannot allocate device memory or bring a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * the same kernels, the same arguments without `workspace`, the same results bit for
+ * bit.  The per-split softmax partials live in a static device array of
+ * DC_ATTN_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the
+ * process ends); a call that needs more -- dc_attn_workspace_bytes(n_b*n_h, group, hd,
+ * n_idx + n_sink + n_recent + 1) -- returns DC_ENOMEM and launches nothing.  The call
+ * allocates and frees nothing.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (two streams, two threads) race; order them on one stream.  The array's
+ * device address is looked up on the first call on each device (a runtime query, no
+ * allocation); make that first call outside graph capture.
+ * No counterpart in the reference, which always allocates through torch.
+ */
+#define DC_ATTN_STATIC_SCRATCH_BYTES (32u << 20)
+int dc_gather_attn_static_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
+                               const void *new_k, const void *new_v, void *out, float *lse, int n_b,
+                               int n_h, int group, int hd, int n_idx, int64_t idx_unit_stride,
+                               const uint32_t *n_idx_unit, int64_t region_lo, int n_sink,
+                               int64_t recent_lo, int n_recent, int64_t k_batch_stride,
+                               int64_t k_head_stride, int64_t k_row_stride, int64_t v_batch_stride,
+                               int64_t v_head_stride, int64_t v_row_stride, float scale, void *stream);
+
+/*
  * k-check (diffcache_cpu/src/nsw.rs:198-296): how many of a unit's best rows are
  * worth attending to.  scores (n_units, scores_unit_stride) fp32: the exact scores of
  * the n_sel selected rows, best first (dc_score_gathered_bf16 on ids in DC_ORDER_BEST
