@@ -28,7 +28,7 @@ SYMBOLS = (
     "dc_version", "dc_last_error", "dc_group_mean_bf16", "dc_score_bf16",
     "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
     "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_gather_attn_static_bf16", "dc_append_kv_bf16",
-    "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
+    "dc_step_advance", "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
     "dc_sparse_select", "dc_score_select_bf16",
@@ -58,6 +58,7 @@ class LayerArgs(C.Structure):
         ("sketch_codes", C.c_void_p), ("sketch_scale", C.c_void_p), ("sketch_resid", C.c_void_p),
         ("sketch_batch_stride", C.c_int64), ("sketch_head_stride", C.c_int64),
         ("sketch_row_stride", C.c_int64),
+        ("n_recent_dev", C.c_void_p),
     ]
 
 
@@ -77,11 +78,12 @@ def _load() -> C.CDLL:
         "dc_topk_select": (i, [p, i64, p, i64, i, i, i, i, i, p, p, sz, p]),
         "dc_gather_rows_bf16": (i, [p, p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, i64, i64, p]),
         "dc_attn_workspace_bytes": (sz, [i, i, i, i]),
-        "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i,
+        "dc_gather_attn_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i, p,
                                     i64, i64, i64, i64, i64, i64, f, p, sz, p]),
-        "dc_gather_attn_static_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i,
+        "dc_gather_attn_static_bf16": (i, [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, p, i64, i, i64, i, p,
                                            i64, i64, i64, i64, i64, i64, f, p]),
-        "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, i64, i64, i64, p]),
+        "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, p, i64, i64, i64, i64, p]),
+        "dc_step_advance": (i, [p, i, i, p]),
         "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
         "dc_layer_workspace_bytes": (sz, [i, i, i, i, i, i]),
         "dc_decode_layer": (i, [C.POINTER(LayerArgs), p]),
@@ -142,6 +144,15 @@ def _opt(t: Optional[torch.Tensor], name: str):
 
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
+
+
+def _counter(t: Optional[torch.Tensor]):
+    """Device pointer of a one-element int32 step counter, or None."""
+    if t is None:
+        return None
+    if not t.is_cuda or t.dtype != torch.int32 or t.numel() < 1:
+        raise DiffCacheError("a step counter must be an int32 tensor in GPU memory")
+    return t.data_ptr()
 
 
 def _store_strides(store: torch.Tensor) -> Tuple[int, int, int]:
@@ -364,9 +375,11 @@ def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
                 new_v: Optional[torch.Tensor] = None, scale: Optional[float] = None,
                 out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                 workspace: Optional[torch.Tensor] = None,
-                n_idx_unit: Optional[torch.Tensor] = None) -> torch.Tensor:
+                n_idx_unit: Optional[torch.Tensor] = None,
+                n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q (b, h*group, hd) bf16 -> out (b, h*group, hd) bf16.  ``n_idx_unit`` (b*h) int32:
-    per-unit number of leading ids to attend to (see ``kcheck``)."""
+    per-unit number of leading ids to attend to (see ``kcheck``).  ``n_recent_dev``: one
+    int32 on the device holding the current suffix length (``n_recent`` is then its capacity)."""
     ksb, ksh, ksr = _store_strides(store_k)
     vsb, vsh, vsr = _store_strides(store_v)
     b, h, _, hd = store_k.shape
@@ -385,8 +398,8 @@ def gather_attn(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor,
         _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v"), _opt(idx, "idx"),
         _opt(new_k, "new_k"), _opt(new_v, "new_v"), _dev(out, "out"), _opt(lse, "lse"), b, h, group,
         hd, n_idx, 0 if idx is None else idx.stride(0), _opt(n_idx_unit, "n_idx_unit"), region_lo, n_sink,
-        recent_lo, n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, _dev(workspace, "workspace"), workspace.numel(),
-        _stream()))
+        recent_lo, n_recent, _counter(n_recent_dev), ksb, ksh, ksr, vsb, vsh, vsr, scale,
+        _dev(workspace, "workspace"), workspace.numel(), _stream()))
     return out
 
 
@@ -395,7 +408,8 @@ def gather_attn_static(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Te
                        n_recent: int, out: torch.Tensor, new_k: Optional[torch.Tensor] = None,
                        new_v: Optional[torch.Tensor] = None, scale: Optional[float] = None,
                        lse: Optional[torch.Tensor] = None,
-                       n_idx_unit: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       n_idx_unit: Optional[torch.Tensor] = None,
+                       n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``gather_attn`` without a workspace and without any allocation (dc_gather_attn_static_bf16):
     the split partials live in a static device array of the library.  q, new_k, new_v must be
     contiguous and ``out`` is the caller's; sizes beyond the array raise DiffCacheError."""
@@ -413,7 +427,7 @@ def gather_attn_static(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Te
         _dev(q, "q"), _dev(store_k, "store_k"), _dev(store_v, "store_v"), _opt(idx, "idx"),
         _opt(new_k, "new_k"), _opt(new_v, "new_v"), _dev(out, "out"), _opt(lse, "lse"), b, h, group,
         hd, n_idx, 0 if idx is None else idx.stride(0), _opt(n_idx_unit, "n_idx_unit"), region_lo, n_sink,
-        recent_lo, n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, _stream()))
+        recent_lo, n_recent, _counter(n_recent_dev), ksb, ksh, ksr, vsb, vsh, vsr, scale, _stream()))
     return out
 
 
@@ -443,7 +457,11 @@ def kcheck(scores: torch.Tensor, n_sel: int, hd: int, k_check_seq, attn_mass_thr
 
 
 def append_kv(store_k: torch.Tensor, store_v: torch.Tensor, new_k: torch.Tensor,
-              new_v: torch.Tensor, pos: int) -> None:
+              new_v: torch.Tensor, pos: int, pos_dev: Optional[torch.Tensor] = None,
+              pos_end: Optional[int] = None) -> None:
+    """store[b, h, pos (+ pos_dev[0]), :] = new_k / new_v[b, h, :]; ``pos_dev``: an int32
+    counter on the device added to ``pos`` when the kernel runs; rows at or beyond
+    ``pos_end`` (default: the store's length) are not written."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
         raise DiffCacheError("K and V stores must share their strides")
@@ -454,8 +472,14 @@ def append_kv(store_k: torch.Tensor, store_v: torch.Tensor, new_k: torch.Tensor,
     if new_k.numel() != b * h * hd or new_v.numel() != b * h * hd:
         raise DiffCacheError("new_k/new_v must hold (b, h, hd) values")
     _check(lib.dc_append_kv_bf16(_dev(store_k, "store_k"), _dev(store_v, "store_v"),
-                                 _dev(new_k, "new_k"), _dev(new_v, "new_v"), b, h, hd, pos, sb, sh, sr,
-                                 _stream()))
+                                 _dev(new_k, "new_k"), _dev(new_v, "new_v"), b, h, hd, pos,
+                                 _counter(pos_dev), n_max if pos_end is None else min(pos_end, n_max),
+                                 sb, sh, sr, _stream()))
+
+
+def step_advance(counter: torch.Tensor, delta: int = 1, limit: int = 2 ** 31 - 1) -> None:
+    """counter[0] = clamp(counter[0] + delta, 0, limit), enqueued on the current stream."""
+    _check(lib.dc_step_advance(_counter(counter), delta, limit, _stream()))
 
 
 def ingest_kv(store: torch.Tensor, src: torch.Tensor, dst_pos: int = 0) -> None:
@@ -486,8 +510,10 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
                  order: int = ORDER_ANY, scale: Optional[float] = None,
                  select_state_ready: bool = False,
                  scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
-                 sketch: Optional["Sketch"] = None) -> torch.Tensor:
+                 sketch: Optional["Sketch"] = None,
+                 n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """score -> select -> attend for one layer, enqueued on the current stream.
+    ``n_recent_dev``: the suffix length as a device-side int32 (``n_recent`` = capacity).
     ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
     ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result)."""
     sb, sh, sr = _store_strides(store_k)
@@ -530,6 +556,7 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
         a.sketch_codes, a.sketch_scale = _dev(c, "codes"), _dev(sketch.scale, "scale")
         a.sketch_resid = _dev(sketch.resid, "resid")
         a.sketch_batch_stride, a.sketch_head_stride, a.sketch_row_stride = c.stride(0), c.stride(1), c.stride(2)
+    a.n_recent_dev = _counter(n_recent_dev)
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
 

@@ -129,7 +129,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     }
     rc = dc_gather_attn_bf16(a->q, a->k, a->v, a->idx_out, a->new_k, a->new_v, a->out, a->lse, a->n_b,
                              a->n_h, a->group, a->hd, k_eff, a->idx_unit_stride, nullptr, a->n_sink, a->n_sink,
-                             a->recent_lo, a->n_recent, a->kv_batch_stride, a->kv_head_stride,
+                             a->recent_lo, a->n_recent, a->n_recent_dev, a->kv_batch_stride, a->kv_head_stride,
                              a->kv_row_stride, a->kv_batch_stride, a->kv_head_stride,
                              a->kv_row_stride, a->scale, w.attn, w.attn_bytes, stream);
     return rc;

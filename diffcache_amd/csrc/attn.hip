@@ -44,8 +44,8 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint32_t *__restrict__ idx, const uint16_t *__restrict__ new_k,
     const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml,
-    const uint32_t *__restrict__ n_idx_unit, int n_h, int n_idx, int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-    int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
+    const uint32_t *__restrict__ n_idx_unit, const int32_t *__restrict__ n_recent_dev, int n_h, int n_idx,
+    int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent, int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
     int64_t vsr, float scale) {
     constexpr int LPR = HD / 8;
     constexpr int NG = kThreads / LPR;  // row groups per block
@@ -61,6 +61,16 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gid = tid / LPR, col = tid % LPR;
     const int r0 = split * ROWS;
+
+    // The length of the recent window may live on the device (the role of cache_seqlens in
+    // base.py:134-142): n_recent is then its capacity, which sized the grid, and the rows
+    // beyond the actual length are masked like any position past the end of the list.
+    if (n_recent_dev) {
+        int c = *n_recent_dev;
+        c = c < 0 ? 0 : (c < n_recent ? c : n_recent);
+        n_total -= n_recent - c;
+        n_recent = c;
+    }
 
     // only the first n_eff selected ids of the unit count when per-unit sizes are given
     int n_eff = n_idx;
@@ -309,14 +319,15 @@ AttnWs carve_attn(void *base, int n_units, int group, int hd, int n_splits) {
 template <int HD>
 int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const uint16_t *k,
                 const uint16_t *v, const uint32_t *idx, const uint16_t *new_k,
-                const uint16_t *new_v, const AttnWs &w, const uint32_t *n_idx_unit, int n_h, int n_idx,
+                const uint16_t *new_v, const AttnWs &w, const uint32_t *n_idx_unit,
+                const int32_t *n_recent_dev, int n_h, int n_idx,
                 int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
                 int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
                 int64_t vsh, int64_t vsr, float scale) {
 #define DC_ATTN_CASE(GG)                                                                           \
     case GG:                                                                                       \
         hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, q, k, v, idx, \
-                           new_k, new_v, w.acc, w.ml, n_idx_unit, n_h, n_idx, idx_stride,                      \
+                           new_k, new_v, w.acc, w.ml, n_idx_unit, n_recent_dev, n_h, n_idx, idx_stride,        \
                            region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, ksb, ksh,    \
                            ksr, vsb, vsh, vsr, scale);                                             \
         return 0;
@@ -348,9 +359,10 @@ namespace {
 int gather_attn_common(const char *who, const void *q, const void *k, const void *v, const uint32_t *idx,
                        const void *new_k, const void *new_v, void *out, float *lse, int n_b, int n_h,
                        int group, int hd, int n_idx, int64_t idx_unit_stride, const uint32_t *n_idx_unit,
-                       int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent, int64_t ksb,
-                       int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
-                       void *workspace, size_t workspace_bytes, void *stream) {
+                       int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
+                       const int32_t *n_recent_dev, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
+                       int64_t vsh, int64_t vsr, float scale, void *workspace, size_t workspace_bytes,
+                       void *stream) {
     DC_REQUIRE(q && k && v && out, "%s: null pointer", who);
     DC_REQUIRE(n_b >= 0 && n_h >= 1 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
                "%s: bad sizes", who);
@@ -387,15 +399,15 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     const uint16_t *nk16 = (const uint16_t *)new_k, *nv16 = (const uint16_t *)new_v;
     uint16_t *o16 = (uint16_t *)out;
     if (hd == 64)
-        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
+        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else if (hd == 128)
-        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
+        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                               plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     else
-        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_h, n_idx,
+        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
                               idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
                               plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
     DC_REQUIRE(rc == 0, "%s: unsupported group %d", who, group);
@@ -423,12 +435,13 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
                                    int n_b, int n_h, int group, int hd, int n_idx,
                                    int64_t idx_unit_stride, const uint32_t *n_idx_unit,
                                    int64_t region_lo, int n_sink,
-                                   int64_t recent_lo, int n_recent, int64_t ksb, int64_t ksh,
+                                   int64_t recent_lo, int n_recent, const int32_t *n_recent_dev,
+                                   int64_t ksb, int64_t ksh,
                                    int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
                                    void *workspace, size_t workspace_bytes, void *stream) {
     return gather_attn_common("dc_gather_attn_bf16", q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group,
                               hd, n_idx, idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo,
-                              n_recent, ksb, ksh, ksr, vsb, vsh, vsr, scale, workspace, workspace_bytes,
+                              n_recent, n_recent_dev, ksb, ksh, ksr, vsb, vsh, vsr, scale, workspace, workspace_bytes,
                               stream);
 }
 
@@ -437,7 +450,7 @@ extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const vo
                                           int n_b, int n_h, int group, int hd, int n_idx,
                                           int64_t idx_unit_stride, const uint32_t *n_idx_unit,
                                           int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-                                          int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
+                                          const int32_t *n_recent_dev, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
                                           int64_t vsr, float scale, void *stream) {
     const char *who = "dc_gather_attn_static_bf16";
     DC_REQUIRE(n_b >= 0 && n_h >= 1 && group >= 1 && group <= 8 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
@@ -477,8 +490,8 @@ extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const vo
     // Every split slot the merge reads is written by the attention kernel of the same call, so
     // nothing has to start at zero; the contents of the previous call are simply overwritten.
     return gather_attn_common(who, q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group, hd, n_idx,
-                              idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo, n_recent, ksb, ksh,
-                              ksr, vsb, vsh, vsr, scale, ptr, kStaticScratchBytes, stream);
+                              idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo, n_recent, n_recent_dev,
+                              ksb, ksh, ksr, vsb, vsh, vsr, scale, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int dc_gather_rows_bf16(const void *k, const void *v, const uint32_t *idx, void *out_k,

@@ -154,8 +154,8 @@ extern "C" int dc_data_layer_insert(dc_data_layer *dl, const void *keys, const v
     DC_REQUIRE(dl->ctx_len < dl->n_max, "%s: the store is full (%lld rows)", who, (long long)dl->n_max);
     int64_t sb, sh, sr;
     strides_of(dl, &sb, &sh, &sr);
-    int rc = dc_append_kv_bf16(dl->k, dl->v, keys, vals, dl->bsz, dl->kv_heads, dl->hd, dl->ctx_len, sb, sh, sr,
-                               stream);
+    int rc = dc_append_kv_bf16(dl->k, dl->v, keys, vals, dl->bsz, dl->kv_heads, dl->hd, dl->ctx_len, nullptr,
+                               dl->n_max, sb, sh, sr, stream);
     if (rc) return rc;
     if (dl->use_sketch) {
         // the first row fits the scales; later rows keep them and can only raise the residual bounds

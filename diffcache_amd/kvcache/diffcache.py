@@ -25,6 +25,23 @@ own attention over ``get_kvcache()``.
 reference: score -> select -> attention straight from the store (one C call),
 replacing the ``flash_attn_with_kvcache`` call of ``base.py:134-142`` as well.
 
+Step state.  The length of the recent window lives in a one-element int32 tensor on the
+device (``step_state``), like the ``cache_seqlens`` tensor the reference hands to
+flash-attn (``base.py:134-142,150-152``): ``decode_attention`` appends at, and attends up
+to, the row that counter names, and advances it after the last layer.  A call captured
+in a HIP graph therefore stays right on every replay; after replays the host's mirror
+(``kvbuf_suffix_len``) is brought up to date with ``advance_host_step``.
+
+Rollover.  The reference never moves tokens out of the recent window into its index
+(``diffcache.py:221`` asserts instead, although ``lib.rs:352-369`` exists for it), so a
+sequence ends after ``kvbuf_suffix_maxlen - kvbuf_suffix_len`` tokens.  Here the rows are
+already in the store, so when the window is full the region boundary simply moves: the
+oldest rows of the window join the retrieval region (their sketch rows are added with the
+fitted scales kept) and the window shrinks back to its initial length.  This is a
+host-side event between two decode steps (``rollover``; ``generation`` counts them):
+graphs captured before it must be captured again, since the region length is a launch
+parameter.
+
 Two options beyond the reference's arguments.  ``key_sketch`` (default on): an
 8-bit sketch of the keys is built at prefill and the scans read it instead of
 the bf16 keys, rescoring only the rows that can still reach the top-k; the ids
@@ -138,6 +155,13 @@ class DiffCache:
         self._attn_ws: Optional[torch.Tensor] = None
         self._prefix0 = kvbuf_prefix_len
         self._suffix0 = kvbuf_suffix_len
+        # device-side length of the recent window (the host mirror is kvbuf_suffix_len)
+        self.step_state = torch.full((1,), kvbuf_suffix_len, device=self.device, dtype=torch.int32)
+        # suffix rows that are present in kstore / vstore: all of them on the native route,
+        # only the prompt's on the hook route (the harness's attention call writes the new
+        # tokens into kbuf / vbuf, as flash_attn_with_kvcache does for the reference)
+        self._store_suffix_rows = kvbuf_suffix_len
+        self.generation = 0           # number of rollovers so far
 
         init_metrics()
 
@@ -147,17 +171,70 @@ class DiffCache:
         return lo, lo + self.retrieval_region_len
 
     def _ensure_workspace(self) -> torch.Tensor:
+        """Scratch for one layer call, sized once for the longest region the store can hold
+        (the region grows at every rollover)."""
         region = self.retrieval_region_len
-        if self._ws is None or self._ws_rows != region:
+        if self._ws is None or self._ws_rows < region:
             n_units = self.batch_size * self.num_kv_heads
-            attended = min(region, self.retrieval_budget) + self.kvbuf_prefix_len + self.kvbuf_suffix_maxlen + 1
+            cap = max(region, self.max_length - self.kvbuf_prefix_len - min(self._suffix0, self.kvbuf_suffix_maxlen))
+            attended = min(cap, self.retrieval_budget) + self.kvbuf_prefix_len + self.kvbuf_suffix_maxlen + 1
             self._ws = hip.alloc_workspace(
-                hip.layer_workspace_bytes(n_units, region, self.retrieval_budget, self.group,
+                hip.layer_workspace_bytes(n_units, cap, self.retrieval_budget, self.group,
                                           self.head_dim, attended), self.device)
-            self._ws_rows = region
+            self._ws_rows = cap
             self._ws_ready = False
             self._hook_ws_ready = False
         return self._ws
+
+    def _set_suffix_len(self, n: int) -> None:
+        self.kvbuf_suffix_len = n
+        self.step_state.fill_(n)
+
+    def advance_host_step(self, steps: int = 1) -> None:
+        """After ``steps`` replays of a captured decode step: bring the host's mirror of the
+        recent-window length up to the device's counter (no synchronisation)."""
+        self.kvbuf_suffix_len += steps
+        self._store_suffix_rows += steps
+        hip.require(self.kvbuf_suffix_len <= self.kvbuf_suffix_maxlen,
+                    "more steps were replayed than the recent window holds; call rollover() in time")
+
+    def window_full(self) -> bool:
+        return self.kvbuf_suffix_len >= self.kvbuf_suffix_maxlen
+
+    def rollover(self) -> int:
+        """Move the oldest rows of the recent window into the retrieval region (see the module
+        docstring).  Host-side, between two decode steps, never under graph capture.  Returns
+        the number of rows moved."""
+        hip.require(not torch.cuda.is_current_stream_capturing(), "rollover() cannot be captured in a graph")
+        keep = min(self._suffix0, self.kvbuf_suffix_maxlen - 1)
+        moved = self.kvbuf_suffix_len - keep
+        if moved <= 0:
+            return 0
+        lo, hi = self._region()
+        p, s, b0 = self.kvbuf_prefix_len, self.kvbuf_suffix_len, self.retrieval_budget
+        hip.require(hi + s <= self.max_length, "store is full")
+        for l in range(self.num_layers):
+            ks, vs = self.kstore[l], self.vstore[l]
+            have = self._store_suffix_rows
+            if have < s:    # hook route: the decoded tokens live in kbuf / vbuf only
+                ks[:, :, hi + have:hi + s].copy_(self.kbuf[l][:, :, b0 + p + have:b0 + p + s])
+                vs[:, :, hi + have:hi + s].copy_(self.vbuf[l][:, :, b0 + p + have:b0 + p + s])
+            if self.key_sketch:
+                first = self.retrieval_region_len == 0       # nothing was sketched yet: fit the scales
+                self.sketch[l].build(ks, hi if not first else lo, moved, keep_scale=not first)
+            # the assembled buffer's suffix = the rows that stay in the window
+            self.kbuf[l][:, :, b0 + p:b0 + p + keep].copy_(ks[:, :, hi + moved:hi + s])
+            self.vbuf[l][:, :, b0 + p:b0 + p + keep].copy_(vs[:, :, hi + moved:hi + s])
+        self.retrieval_region_len += moved
+        self._set_suffix_len(keep)
+        self._store_suffix_rows = keep
+        self._ws_ready = False
+        self._hook_ws_ready = False
+        self.generation += 1
+        for l in range(self.num_layers):
+            if self.data_layers[l] is not None:
+                self._bind_data_layer(l)
+        return moved
 
     # ------------------------------------------------------------------ prefill
     def prefill_update_kv_cache(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int):
@@ -177,7 +254,8 @@ class DiffCache:
         prefix_len = min(self._prefix0, seq_len)                    # diffcache.py:163
         suffix_len = min(self._suffix0, seq_len - prefix_len)       # diffcache.py:169
         self.kvbuf_prefix_len = prefix_len
-        self.kvbuf_suffix_len = suffix_len
+        self._set_suffix_len(suffix_len)
+        self._store_suffix_rows = suffix_len
         self.retrieval_region_len = seq_len - prefix_len - suffix_len
         if self.key_sketch and self.retrieval_region_len > 0:
             self.sketch[layer_idx].build(self.kstore[layer_idx], prefix_len, self.retrieval_region_len)
@@ -221,6 +299,8 @@ class DiffCache:
     def decode_query_kvcache(self, layer_idx: int) -> None:
         """Exact scan + top-k of the retrieval region with the mean query
         (diffcache.py:211-223 -> lib.rs:373-404 -> nsw.rs:592-630)."""
+        if layer_idx == 0 and self.window_full():
+            self.rollover()                                                  # diffcache.py:221 asserts instead
         retrieval_len = min(self.retrieval_region_len, self.retrieval_budget)
         if retrieval_len > 0:
             lo, hi = self._region()
@@ -238,7 +318,8 @@ class DiffCache:
         hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,
                     "the recent window is full (kvbuf_suffix_maxlen)")       # diffcache.py:221
         if layer_idx == self.num_layers - 1:
-            self.kvbuf_suffix_len += 1
+            self.kvbuf_suffix_len += 1                                       # diffcache.py:222-223
+            hip.step_advance(self.step_state, 1, self.kvbuf_suffix_maxlen)
 
     def decode_post_query_operation(self, layer_idx: int) -> None:
         """Selected rows into kbuf/vbuf[:, :, budget - len : budget] (diffcache.py:196-209)."""
@@ -262,38 +343,48 @@ class DiffCache:
         (bsz, 1, Hkv, hd).  Returns (bsz, Hq, hd) bf16.  Call it for every layer of
         a step; the suffix grows by one after the last layer."""
         b, hq, hkv, hd = self.batch_size, self.num_q_heads, self.num_kv_heads, self.head_dim
+        capturing = torch.cuda.is_current_stream_capturing()
+        if layer_idx == 0 and self.window_full() and not capturing:
+            self.rollover()                                                  # diffcache.py:221 asserts instead
         hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,
-                    "the recent window is full (kvbuf_suffix_maxlen)")       # diffcache.py:221
+                    "the recent window is full (kvbuf_suffix_maxlen): call rollover() between steps")
         lo, hi = self._region()
-        pos = hi + self.kvbuf_suffix_len
-        hip.require(pos < self.max_length, "store is full")
+        hip.require(hi + self.kvbuf_suffix_len < self.max_length, "store is full")
         q = queries.reshape(b, hq, hd)
         if not q.is_contiguous():
             q = q.contiguous()
-        hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], key_states.reshape(b, hkv, hd),
-                      value_states.reshape(b, hkv, hd), pos)
+        nk, nv = key_states.reshape(b, hkv, hd), value_states.reshape(b, hkv, hd)
+        if not nk.is_contiguous():
+            nk = nk.contiguous()
+        if not nv.is_contiguous():
+            nv = nv.contiguous()
+        # the token's row: hi + (device-side window length); never past the window's capacity
+        hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], nk, nv, hi, pos_dev=self.step_state,
+                      pos_end=min(hi + self.kvbuf_suffix_maxlen, self.max_length))
         if out is None:
             if self._attn_out is None:
                 self._attn_out = torch.empty((b, hq, hd), device=self.device, dtype=torch.bfloat16)
             out = self._attn_out
         ws = self._ensure_workspace()
         if self.use_k_check and min(hi - lo, self.retrieval_budget) > 0:
-            self._decode_attention_k_check(layer_idx, q, out, ws)
-            if layer_idx == self.num_layers - 1:
-                self.kvbuf_suffix_len += 1
-            return out
-        hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
-                         self.kvbuf_suffix_len + 1, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
-                         mode=self.mode, order=order, select_state_ready=self._ws_ready,
-                         sketch=self.sketch[layer_idx])
-        self._ws_ready = True
-        self._hook_ws_ready = False
+            self._decode_attention_k_check(layer_idx, q, nk, nv, out, ws)
+        else:
+            # attended: [selected | prefix | the window's rows before this token | this token]
+            hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
+                             self.kvbuf_suffix_maxlen, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
+                             nk, nv, mode=self.mode, order=order, select_state_ready=self._ws_ready,
+                             sketch=self.sketch[layer_idx], n_recent_dev=self.step_state)
+            self._ws_ready = True
+            self._hook_ws_ready = False
         if layer_idx == self.num_layers - 1:
-            self.kvbuf_suffix_len += 1
+            hip.step_advance(self.step_state, 1, self.kvbuf_suffix_maxlen)
+            if not capturing:       # a captured step is counted when it is replayed (advance_host_step)
+                self.kvbuf_suffix_len += 1
+                self._store_suffix_rows += 1
         return out
 
-    def _decode_attention_k_check(self, layer_idx: int, q: torch.Tensor, out: torch.Tensor,
-                                  ws: torch.Tensor) -> None:
+    def _decode_attention_k_check(self, layer_idx: int, q: torch.Tensor, nk: torch.Tensor, nv: torch.Tensor,
+                                  out: torch.Tensor, ws: torch.Tensor) -> None:
         """select (best first) -> exact scores of the selected rows -> k-check -> attention over
         the leading n_eff rows of every unit plus the always-kept rows."""
         lo, hi = self._region()
@@ -316,13 +407,12 @@ class DiffCache:
         hip.score_gathered(ks, self.qbuf, idx[:, :n_sel], row_offset=lo, scores=self._kc_scores)
         hip.kcheck(self._kc_scores, n_sel, self.head_dim, self.k_check_seq, self.attn_mass_threshold,
                    self.mode, n_eff=self.n_eff[layer_idx])
-        n_recent = self.kvbuf_suffix_len + 1
         need = hip.lib.dc_attn_workspace_bytes(n_units, self.group, self.head_dim,
                                                n_sel + self.kvbuf_prefix_len + self.kvbuf_suffix_maxlen + 1)
         if self._attn_ws is None or self._attn_ws.numel() < need:
             self._attn_ws = hip.alloc_workspace(need, self.device)
-        hip.gather_attn(q, ks, vs, idx, n_sel, lo, lo, hi, n_recent, out=out, workspace=self._attn_ws,
-                        n_idx_unit=self.n_eff[layer_idx])
+        hip.gather_attn(q, ks, vs, idx, n_sel, lo, lo, hi, self.kvbuf_suffix_maxlen, nk, nv, out=out,
+                        workspace=self._attn_ws, n_idx_unit=self.n_eff[layer_idx], n_recent_dev=self.step_state)
 
     # ------------------------------------------------------------------ prefill cache
     def save_prefill_cache(self, prefill_cache_path: str) -> None:
@@ -337,6 +427,7 @@ class DiffCache:
         with open(path, "w") as f:
             json.dump(metadata, f)
         b0, p, s = self.retrieval_budget, self.kvbuf_prefix_len, self.kvbuf_suffix_len
+        _, hi = self._region()
         for layer_idx in range(self.num_layers):
             layer_path = os.path.join(prefill_cache_path, f"p_l_{layer_idx:03d}")
             os.makedirs(layer_path, exist_ok=False)
@@ -345,8 +436,15 @@ class DiffCache:
         for layer_idx in range(self.num_layers):
             layer_path = os.path.join(prefill_cache_path, f"s_l_{layer_idx:03d}")
             os.makedirs(layer_path, exist_ok=False)
-            torch.save(self.kbuf[layer_idx][:, :, b0 + p:b0 + p + s, :], os.path.join(layer_path, "k.pt"))
-            torch.save(self.vbuf[layer_idx][:, :, b0 + p:b0 + p + s, :], os.path.join(layer_path, "v.pt"))
+            # The window's rows: from the store where it has them (the native route appends
+            # there and never touches kbuf / vbuf), else from the assembled buffer (hook route).
+            have = min(self._store_suffix_rows, s)
+            sk = torch.cat([self.kstore[layer_idx][:, :, hi:hi + have],
+                            self.kbuf[layer_idx][:, :, b0 + p + have:b0 + p + s]], dim=2)
+            sv = torch.cat([self.vstore[layer_idx][:, :, hi:hi + have],
+                            self.vbuf[layer_idx][:, :, b0 + p + have:b0 + p + s]], dim=2)
+            torch.save(sk, os.path.join(layer_path, "k.pt"))
+            torch.save(sv, os.path.join(layer_path, "v.pt"))
         for layer_idx in range(self.num_layers):
             layer_path = os.path.join(prefill_cache_path, f"d_l_{layer_idx:03d}")
             os.makedirs(layer_path, exist_ok=False)
@@ -359,7 +457,8 @@ class DiffCache:
             metadata = json.load(f)
         self.r_sq = metadata["r_sq"]
         self.kvbuf_prefix_len = metadata["kvbuf_prefix_len"]
-        self.kvbuf_suffix_len = metadata["kvbuf_suffix_len"]
+        self._set_suffix_len(metadata["kvbuf_suffix_len"])
+        self._store_suffix_rows = self.kvbuf_suffix_len
         self.retrieval_region_len = metadata["retrieval_region_len"]
         b0, p, s = self.retrieval_budget, self.kvbuf_prefix_len, self.kvbuf_suffix_len
         lo, hi = self._region()

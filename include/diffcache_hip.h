@@ -203,6 +203,11 @@ size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attend
  * n_idx_unit: NULL, or (n_b*n_h) uint32: unit u attends only to its first
  * min(n_idx_unit[u], n_idx) retrieved rows (the output of dc_kcheck_f32 on ids in
  * DC_ORDER_BEST order); the always-kept rows are unaffected.
+ * n_recent_dev: NULL, or one int32 in device memory holding the current length of the
+ * suffix: the kernels then attend to min(*n_recent_dev, n_recent) suffix rows and n_recent
+ * is the capacity that sizes the launch and the workspace.  This is what keeps a call that
+ * was captured in a graph valid on later replays, as the cache_seqlens tensor does for
+ * flash_attn_with_kvcache (src/diffcache/base.py:134-142,150-152); dc_step_advance moves it.
  * Replaces flash_attn_with_kvcache over the assembled buffer
  * (src/diffcache/base.py:134-142) and the buffer assembly it reads
  * (src/diffcache/kvcache/diffcache.py:48-66,186-209).
@@ -211,10 +216,10 @@ int dc_gather_attn_bf16(const void *q, const void *k, const void *v, const uint3
                         const void *new_k, const void *new_v, void *out, float *lse, int n_b,
                         int n_h, int group, int hd, int n_idx, int64_t idx_unit_stride,
                         const uint32_t *n_idx_unit, int64_t region_lo, int n_sink, int64_t recent_lo,
-                        int n_recent, int64_t k_batch_stride, int64_t k_head_stride,
-                        int64_t k_row_stride, int64_t v_batch_stride, int64_t v_head_stride,
-                        int64_t v_row_stride, float scale, void *workspace, size_t workspace_bytes,
-                        void *stream);
+                        int n_recent, const int32_t *n_recent_dev, int64_t k_batch_stride,
+                        int64_t k_head_stride, int64_t k_row_stride, int64_t v_batch_stride,
+                        int64_t v_head_stride, int64_t v_row_stride, float scale, void *workspace,
+                        size_t workspace_bytes, void *stream);
 
 /*
  * dc_gather_attn_bf16 for callers that cannot allocate device memory or bring a workspace
@@ -235,9 +240,10 @@ int dc_gather_attn_static_bf16(const void *q, const void *k, const void *v, cons
                                const void *new_k, const void *new_v, void *out, float *lse, int n_b,
                                int n_h, int group, int hd, int n_idx, int64_t idx_unit_stride,
                                const uint32_t *n_idx_unit, int64_t region_lo, int n_sink,
-                               int64_t recent_lo, int n_recent, int64_t k_batch_stride,
-                               int64_t k_head_stride, int64_t k_row_stride, int64_t v_batch_stride,
-                               int64_t v_head_stride, int64_t v_row_stride, float scale, void *stream);
+                               int64_t recent_lo, int n_recent, const int32_t *n_recent_dev,
+                               int64_t k_batch_stride, int64_t k_head_stride, int64_t k_row_stride,
+                               int64_t v_batch_stride, int64_t v_head_stride, int64_t v_row_stride,
+                               float scale, void *stream);
 
 /*
  * k-check (diffcache_cpu/src/nsw.rs:198-296): how many of a unit's best rows are
@@ -259,14 +265,26 @@ int dc_kcheck_f32(const float *scores, int64_t scores_unit_stride, int n_units, 
                   uint32_t *n_eff, float *alpha_out, float *mass_out, void *stream);
 
 /*
- * Append one token: k_store[b, h, pos, :] = new_k[b, h, :] (same for v).
+ * Append one token: k_store[b, h, row, :] = new_k[b, h, :] (same for v), row = pos, or
+ * pos + *pos_dev when pos_dev (one int32 in device memory) is not NULL -- the position
+ * then moves with the device-side step count, so a captured call stays valid across
+ * replays.  Rows outside [0, pos_end) are never written (pos itself must be inside).
  * new_k/new_v (n_b, n_h, hd) contiguous.
  * Replaces DataLayer::insert / Index::insert's row write
  * (diffcache_cpu/src/lib.rs:352-369, nsw.rs:551-557); no graph is built.
  */
 int dc_append_kv_bf16(void *k_store, void *v_store, const void *new_k, const void *new_v, int n_b,
-                      int n_h, int hd, int64_t pos, int64_t batch_stride, int64_t head_stride,
-                      int64_t row_stride, void *stream);
+                      int n_h, int hd, int64_t pos, const int32_t *pos_dev, int64_t pos_end,
+                      int64_t batch_stride, int64_t head_stride, int64_t row_stride, void *stream);
+
+/*
+ * *counter = clamp(*counter + delta, 0, limit), enqueued on `stream` (one thread).  The
+ * device-side step count that dc_append_kv_bf16 (pos_dev) and the attention entry points
+ * (n_recent_dev) read: advance it once per decoded token, after the last layer, as the
+ * reference advances kvbuf_suffix_len (src/diffcache/kvcache/diffcache.py:221-223) and
+ * its cache_seqlens (src/diffcache/base.py:150-152).
+ */
+int dc_step_advance(int32_t *counter, int delta, int limit, void *stream);
 
 /*
  * Prefill ingest: src (n_b, seq, n_h, hd) -> store[b, h, dst_pos + s, :].
@@ -320,6 +338,8 @@ typedef struct dc_layer_args {
     const float *sketch_scale;   /* (n_b*n_h, hd) */
     const float *sketch_resid;   /* (n_b*n_h, hd) */
     int64_t sketch_batch_stride, sketch_head_stride, sketch_row_stride; /* bytes */
+    const int32_t *n_recent_dev; /* NULL, or the device-side length of the suffix (see
+                             dc_gather_attn_bf16): n_recent is then its capacity */
 } dc_layer_args;
 
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,

@@ -36,7 +36,7 @@ def _static_call(hip, k, v, q, nk, nv, idx, n_unit, lo, hi, sink, recent, out, l
     p = lambda t: None if t is None else t.data_ptr()
     return hip.lib.dc_gather_attn_static_bf16(
         p(q), p(k), p(v), p(idx), p(nk), p(nv), p(out), p(lse), b, h, grp, hd, idx.shape[1], idx.stride(0),
-        p(n_unit), lo, sink, hi, recent, k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1),
+        p(n_unit), lo, sink, hi, recent, None, k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1),
         v.stride(2), 1.0 / math.sqrt(hd), torch.cuda.current_stream().cuda_stream)
 
 
@@ -80,7 +80,7 @@ def test_static_scratch_attention_rejects_sizes_beyond_its_scratch():
     need = hip.lib.dc_attn_workspace_bytes(b * h, grp, hd, 1024 + 4 + 64 + 1)
     assert need > (32 << 20)
     rc = hip.lib.dc_gather_attn_static_bf16(
-        p(q), p(k), p(k), p(idx), None, None, p(out), None, b, h, grp, hd, 1024, 1024, None, 4, 4, 4, 0,
+        p(q), p(k), p(k), p(idx), None, None, p(out), None, b, h, grp, hd, 1024, 1024, None, 4, 4, 4, 0, None,
         0, 0, hd, 0, 0, hd, 0.1, torch.cuda.current_stream().cuda_stream)
     assert rc == -12, rc
     msg = hip.lib.dc_last_error().decode()
