@@ -1,29 +1,32 @@
 #!/usr/bin/env python3
 """Benchmark of the decode-time retrieval path on one MI355X.
 
-Workload (default): benchmark configuration 3 -- a full 32-layer Llama-3-8B-shaped
-decode step, batch 8, context 131072 per sequence, 32 query / 8 kv heads,
-head_dim 128, bf16 K/V resident in HBM (~137 GB), top-k 2048 plus 4 sink tokens
-and a 64-token recent window.  One "step" = for every layer: score the whole
-retrieval region with the GQA-mean query, select the exact top-k, run the
-gathered attention (including the current token's k/v).  Inputs are synthetic
-and already in HBM when the timed region starts.
+Headline workload: benchmark configuration 3 -- a full 32-layer Llama-3-8B-shaped decode
+step, batch 8, context 131072 per sequence, 32 query / 8 kv heads, head_dim 128, bf16 K/V
+resident in HBM (~137 GB), top-k 2048 plus 4 sink tokens and a 64-token recent window.
+One "step" = for every layer: score the whole retrieval region with the GQA-mean query,
+select the exact top-k, run the gathered attention (including the current token's k/v).
+Inputs are synthetic and already in HBM when the timed region starts.
 
-By default the scan reads the 8-bit sketch of the keys and rescans the rows that can
-still reach the top-k from the bf16 keys (same ids); --scan bf16 streams the bf16
-keys themselves.
+Two scan routes give the same ids: "sketch" (default) scans an 8-bit sketch of the keys
+and rescans the rows that can still reach the top-k from the bf16 keys; "bf16" streams
+the bf16 keys themselves, which is the byte count of the reference's algorithm
+(every key row once).  A default run times both on configuration 3 and, beside it,
+configurations 2 (one layer, 32K context), 5 (1M context) and 4 (PQ baseline).
 
-Prints ONE JSON line.  `value` is the latency of one whole decode step in
-microseconds (lower is better); `roofline` describes the scan kernel (bytes it must
-stream per launch over its measured duration, against the 8 TB/s HBM peak);
-`cpu_baseline` is the C restatement of the reference's exact scan timed on this
-machine's host cores.
+Prints ONE JSON line.  `value` is the latency of one whole decode step of configuration 3
+on the default route, in microseconds (lower is better).  `roofline` describes that route's
+scan kernel: bytes it must stream per launch over its measured duration, against the
+8 TB/s HBM peak (`frac`), and the same duration priced at the two bytes per key element of
+the reference's algorithm (`frac_8d`, which can exceed 1 because the sketch reads one).
+`routes.bf16` is the same step streaming the bf16 keys; `configs` holds the other
+configurations; `cpu_baseline` is the C restatement of the reference's exact scan timed on
+this machine's host cores.
 """
 from __future__ import annotations
 
 import argparse
 import json
-import math
 import os
 import sys
 import time
@@ -33,27 +36,30 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one scan launch of config 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE scaled
-# by a known-size copy kernel (the figures and commands are kept with the other profile
-# summaries of this repository): counts x 2 KiB read + counts x 1 KiB written.
-SCAN_TRAFFIC_BYTES_C3 = {"sketch": 524_722 * 2048 + 13_249 * 1024,
-                         "bf16": 1_053_933 * 2048 + 12_570 * 1024}
+# HBM bytes one scan launch of configuration 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# scaled by a known-size copy kernel: counts x 2 KiB read + counts x 1 KiB written.  Taken
+# once, when the profile summaries kept with this repository were made -- not in this run.
+SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_722 * 2048 + 13_249 * 1024,
+                            "bf16": 1_053_933 * 2048 + 12_570 * 1024}
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
-    "c3": dict(layers=32, batch=8, hq=32, hkv=8, hd=128, ctx=131072, budget=2048, sink=4, recent=64,
+    "c3": dict(id=3, layers=32, batch=8, hq=32, hkv=8, hd=128, ctx=131072, budget=2048, sink=4, recent=64,
                desc="config3: 32-layer Llama-3-8B-shaped decode step, batch 8, ctx 131072, "
                     "32q/8kv heads, hd 128, bf16 K/V in HBM, top-k 2048 + 4 sinks + 64 recent"),
-    "c2": dict(layers=1, batch=1, hq=32, hkv=8, hd=128, ctx=32768, budget=1024, sink=4, recent=64,
+    "c2": dict(id=2, layers=1, batch=1, hq=32, hkv=8, hd=128, ctx=32768, budget=1024, sink=4, recent=64,
                desc="config2: one Llama-3-8B-shaped decode layer, batch 1, ctx 32768, "
                     "top-k 1024 + 4 sinks + 64 recent"),
-    "c5": dict(layers=32, batch=1, hq=32, hkv=8, hd=128, ctx=1048576, budget=4096, sink=4, recent=64,
+    "c5": dict(id=5, layers=32, batch=1, hq=32, hkv=8, hd=128, ctx=1048576, budget=4096, sink=4, recent=64,
                desc="config5: 32 layers, batch 1, ctx 1048576, top-k 4096 + 4 sinks + 64 recent"),
 }
+C4_DESC = ("config4: PQ baseline, 8 kv heads x 1048576 keys, hd 128, M 32 x 256 centroids, "
+           "ADC scan -> 4096 candidates -> exact rerank to top-k 1024")
 
 
 def algorithmic_bytes_per_unit(n_region: int, attended: int, group: int, hd: int) -> int:
-    """K streamed once + gathered K and V rows + q in / out (bf16)."""
+    """Bytes of the reference's algorithm per (layer, batch, kv-head) unit and decode step:
+    K streamed once + gathered K and V rows + q in / out (bf16)."""
     return n_region * hd * 2 + 2 * attended * hd * 2 + group * hd * 2 * 2
 
 
@@ -103,48 +109,6 @@ def make_layer(torch, cfg, layer: int, cfg_id: int, dev, k, v):
     return k, v, q.contiguous(), new_k, new_v
 
 
-def cpu_baseline(torch, cfg, layers_data, target_s: float = 10.0):
-    """The C restatement of the reference's exact-scan path, timed on this box's
-    host cores on a bounded sample: layer 0, batch element 0 (hkv units), one
-    thread per unit like rayon's fan-out, repeated until ~target_s of work."""
-    import numpy as np
-    from oracle import cpu_ref
-    k, v, q, nk, nv = layers_data[0]
-    hkv, hq, hd, n = cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"]
-    grp = hq // hkv
-
-    def host(t):
-        return t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
-
-    k0, v0 = host(k[0]), host(v[0])                       # (hkv, n, hd)
-    q0 = host(q[0]).reshape(hkv, grp, hd)
-    nk0, nv0 = host(nk[0]), host(nv[0])
-    cores = os.cpu_count() or 1
-    # the GPU box gives one GPU's share of the host: 16 cores
-    threads = min(hkv, cores, 16)
-    cpu_ref.lib()
-    reps, total = 0, 0.0
-    t_first = None
-    while total < target_s and reps < 20000:
-        t0 = time.perf_counter()
-        cpu_ref.decode_layer(q0, k0, v0, cfg["budget"], cfg["sink"], cfg["recent"], n_ctx=n,
-                             new_k_u16=nk0, new_v_u16=nv0, n_threads=threads, want_ids=False)
-        dt = time.perf_counter() - t0
-        t_first = dt if t_first is None else t_first
-        total += dt
-        reps += 1
-    per_sample = total / reps
-    units_total = cfg["layers"] * cfg["batch"] * hkv
-    step_us = per_sample * (units_total / hkv) * 1e6
-    return {
-        "value": step_us, "unit": "us", "cores": threads, "kind": "port",
-        "sample": (f"oracle/cpu_ref.c decode_layer on layer 0, batch element 0 ({hkv} units x {n} rows), "
-                   f"{threads} threads, mean of {reps} runs = {per_sample * 1e3:.1f} ms; scaled x"
-                   f"{units_total // hkv} to the full step ({cfg['layers']} layers x batch {cfg['batch']}); "
-                   f"host reports {cores} cpus"),
-    }
-
-
 def make_pq_index(torch, hip, dev, store=None):
     """Benchmark configuration 4: 8 kv heads x 1,048,576 keys ~ N(0,1), hd 128, M 32 x 256 centroids
     from seeded k-means on a 65,536-key sample, 8-bit codes, 4096 candidates, top-k 1024.
@@ -160,30 +124,218 @@ def make_pq_index(torch, hip, dev, store=None):
     return index, store, q
 
 
-def run_pq(args, torch, hip, dev) -> int:
-    """Benchmark configuration 4: PQ baseline, one layer, 8 kv heads x 1,048,576 keys, M 32 x 8-bit
-    codes, ADC scan -> 4096 candidates -> exact bf16 rerank to top-k 1024."""
-    h, n, hd, m, n_cand, topk = 8, 1 << 20, 128, 32, 4096, 1024
+class Slabs:
+    """One allocation for every layer's values, one for the keys, one for the 8-bit key sketch,
+    as diffcache_amd.DiffCache lays its store out (scans of one large allocation run about 3 %
+    faster on MI355X than scans of per-layer allocations; the sketch, which every step streams,
+    is allocated last).  Configurations of equal size (3 and 5) reuse them."""
+
+    def __init__(self, torch, dev, numel: int, sketch: bool):
+        self.v = torch.empty((numel,), dtype=torch.bfloat16, device=dev)
+        self.k = torch.empty((numel,), dtype=torch.bfloat16, device=dev)
+        self.c = torch.empty((numel,), dtype=torch.uint8, device=dev) if sketch else None
+        self.numel = numel
+
+
+class DecodeWorkload:
+    """The data of one configuration in HBM, and timed decode steps over it."""
+
+    def __init__(self, torch, hip, name: str, dev, slabs: Slabs = None, sketch: bool = True):
+        self.torch, self.hip, self.name, self.dev = torch, hip, name, dev
+        cfg = self.cfg = CONFIGS[name]
+        L, b, hkv, n, hd = cfg["layers"], cfg["batch"], cfg["hkv"], cfg["ctx"], cfg["hd"]
+        numel = L * b * hkv * n * hd
+        if slabs is None or slabs.numel < numel:
+            slabs = Slabs(torch, dev, numel, sketch)
+        shape = (L, b, hkv, n, hd)
+        t0 = time.perf_counter()
+        kslab, vslab = slabs.k[:numel].view(shape), slabs.v[:numel].view(shape)
+        self.layers = [make_layer(torch, cfg, l, cfg["id"], dev, kslab[l], vslab[l]) for l in range(L)]
+        self.lo, self.hi = cfg["sink"], n - cfg["recent"]
+        self.region = self.hi - self.lo
+        self.sketches = None
+        if sketch and slabs.c is not None:
+            # the sketch of the retrieval region of every layer (prefill-time work, untimed)
+            cslab = slabs.c[:numel].view(shape)
+            self.sketches = [hip.Sketch(kslab[l], codes=cslab[l]).build(kslab[l], self.lo, self.region)
+                             for l in range(L)]
+        torch.cuda.synchronize()
+        self.setup_s = time.perf_counter() - t0
+        self.n_units = b * hkv
+        self.grp = cfg["hq"] // hkv
+        self.k_eff = min(cfg["budget"], self.region)
+        self.attended = self.k_eff + cfg["sink"] + cfg["recent"] + 1
+        nu, budget = self.n_units, cfg["budget"]
+        self.idx = torch.empty((nu, budget), dtype=torch.int32, device=dev)
+        self.out = torch.empty((b, cfg["hq"], hd), dtype=torch.bfloat16, device=dev)
+        self.ws = hip.alloc_workspace(hip.layer_workspace_bytes(nu, self.region, budget, self.grp, hd,
+                                                                self.attended), dev)
+        self.scores = None
+        self.stream = torch.cuda.Stream(device=dev)     # default priority
+        self.clean = False
+
+    def layer(self, l: int, scan: str, mode: int, ev=None):
+        """One dc_decode_layer call.  scan: "sketch", "bf16" or "dense" (fp32 scores +
+        dc_topk_select).  ev: an event pair recorded around the scan kernel."""
+        hip, cfg = self.hip, self.cfg
+        k, v, q, nk, nv = self.layers[l]
+        if scan == "dense" and self.scores is None:
+            self.scores = self.torch.empty((self.n_units, self.region), dtype=self.torch.float32, device=self.dev)
+        hip.decode_layer(q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
+                         self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv,
+                         mode=mode, order=hip.ORDER_ANY,
+                         select_state_ready=self.clean and scan != "dense", scan_events=ev,
+                         sketch=self.sketches[l] if scan == "sketch" else None)
+        self.clean = scan != "dense"
+
+    def measure(self, scan: str, mode: int, steps: int, warmup: int, event_stride: int = 4,
+                graph: bool = False, cold: bool = False) -> dict:
+        torch, cfg = self.torch, self.cfg
+        L = cfg["layers"]
+        if scan == "sketch" and self.sketches is None:
+            raise RuntimeError("this workload was built without a sketch")
+        timed = list(range(0, L, max(1, event_stride)))
+
+        def new_events(count):
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+            for e in evs:       # torch creates the native event on first record; the C side needs the handle
+                e.record(self.stream)
+            return evs
+
+        def step(evs):
+            with torch.cuda.stream(self.stream):
+                for l in range(L):
+                    ev = None
+                    if evs is not None and l in timed:
+                        j = timed.index(l)
+                        ev = (evs[2 * j], evs[2 * j + 1])
+                    self.layer(l, scan, mode, ev)
+
+        events = [new_events(2 * len(timed)) for _ in range(steps)]
+        marks = new_events(steps + 1)
+        torch.cuda.synchronize()
+        for _ in range(warmup):
+            step(None)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        marks[0].record(self.stream)
+        for s in range(steps):
+            step(events[s])
+            marks[s + 1].record(self.stream)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        ms_per_step = elapsed * 1e3 / steps
+        per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(steps))
+
+        def pct(p):
+            return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
+
+        sc = [e[2 * j].elapsed_time(e[2 * j + 1]) for e in events for j in range(len(timed))]
+        scan_ms = sum(sc) / len(sc)
+
+        # Small configurations fit in the 256 MB Infinity Cache, so the loop above measures a warm
+        # cache.  Cold: a 1 GiB buffer is overwritten before every step (untimed) and each step is
+        # timed on its own.
+        cold_us = None
+        if cold:
+            flush = torch.empty((1 << 30,), dtype=torch.uint8, device=self.dev)
+            c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            samples = []
+            for s_i in range(min(steps, 30)):
+                with torch.cuda.stream(self.stream):
+                    flush.fill_(s_i & 0xff)
+                    c0.record()
+                step(None)
+                with torch.cuda.stream(self.stream):
+                    c1.record()
+                torch.cuda.synchronize()
+                samples.append(c0.elapsed_time(c1) * 1e3)
+            samples.sort()
+            cold_us = samples[len(samples) // 2]
+            del flush
+
+        graph_us = None
+        if graph:
+            # every call of the step only enqueues kernels, so the whole step can be captured; the
+            # select state is already "left ready" by the eager steps above
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=self.stream):
+                for l in range(L):
+                    self.layer(l, scan, mode, None)
+            torch.cuda.synchronize()
+            for _ in range(max(warmup, 1)):
+                g.replay()
+            torch.cuda.synchronize()
+            tg = time.perf_counter()
+            for _ in range(steps):
+                g.replay()
+            torch.cuda.synchronize()
+            graph_us = (time.perf_counter() - tg) * 1e6 / steps
+
+        hd, nu = cfg["hd"], self.n_units
+        unit_bytes = algorithmic_bytes_per_unit(self.region, self.k_eff + cfg["sink"] + cfg["recent"], self.grp, hd)
+        step_bytes = unit_bytes * nu * L                      # the reference's algorithm
+        # what this route has to move: the sketch scan reads hd bytes per key, not 2 * hd
+        path_bytes = step_bytes - (nu * L * self.region * hd if scan == "sketch" else 0)
+        rows_bytes_8d = nu * self.region * hd * 2             # one launch, every bf16 key row once
+        scan_bytes = rows_bytes_8d // 2 if scan == "sketch" else rows_bytes_8d + \
+            (nu * self.region * 4 if scan == "dense" else 0)
+        ach = scan_bytes / (scan_ms * 1e-3) / 1e9
+        roofline = {
+            "bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBPS,
+            "traffic": None,
+            "kernel": {"sketch": "sketch_prune_kernel<128>", "bf16": "score_prune_kernel<128>",
+                       "dense": "score_kernel<128>"}[scan],
+            "algorithmic_bytes_per_launch": scan_bytes, "avg_launch_us": scan_ms * 1e3,
+            "timed_launches": len(sc),
+            # the same launch priced at the reference algorithm's bytes (two per key element)
+            "achieved_8d": rows_bytes_8d / (scan_ms * 1e-3) / 1e9,
+            "frac_8d": rows_bytes_8d / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        }
+        if self.name == "c3" and scan in SCAN_TRAFFIC_PROFILED_C3:
+            roofline["traffic"] = SCAN_TRAFFIC_PROFILED_C3[scan]
+            roofline["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE when the committed profile " \
+                                         "summaries were taken, not measured in this run"
+        s_per_step = ms_per_step * 1e-3
+        return {
+            "value": ms_per_step * 1e3, "unit": "us", "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
+            "workload": cfg["desc"], "scan": scan,
+            "call_path": "dc_decode_layer" + {"sketch": " (sketch scan + exact rescoring)", "bf16": "",
+                                              "dense": " (dense scores)"}[scan],
+            "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
+            "roofline": roofline,
+            # bytes this route must move per step over the step time: the step-level HBM fraction
+            "step_path_bytes": path_bytes,
+            "step_path_gbps": path_bytes / s_per_step / 1e9,
+            "step_path_frac": path_bytes / s_per_step / 1e9 / HBM_PEAK_GBPS,
+            # bytes of the reference's algorithm (every bf16 key once + gathered rows) over the same time
+            "step_8d_bytes": step_bytes,
+            "step_8d_gbps": step_bytes / s_per_step / 1e9,
+            "step_8d_frac": step_bytes / s_per_step / 1e9 / HBM_PEAK_GBPS,
+            "keys_scored_per_s": nu * L * self.region / s_per_step,
+            "cold_cache_step_us_median": cold_us,
+            "graph_step_us": graph_us,
+        }
+
+
+def measure_pq(torch, hip, dev, steps: int, warmup: int, stepwise: bool = False, store=None) -> dict:
+    """Benchmark configuration 4: tables + ADC scan -> 4096 candidates -> exact bf16 rerank -> top 1024."""
+    h, n, m, n_cand, topk = 8, 1 << 20, 32, 4096, 1024
     t_gen = time.perf_counter()
-    index, store, q = make_pq_index(torch, hip, dev)
+    index, store, q = make_pq_index(torch, hip, dev, store)
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t_gen
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps)]
-
-    def step(e=None):
-        if args.stepwise:
-            return step_stepwise(e)
-        lut = hip.pq_build_lut(q, index.books, 1)
-        ids = hip.pq_search(store, index.codes, lut, q, n_cand, topk, idx_out=index.ids,
-                            workspace=index.ws, state_ready=index._ws_ready, scan_events=e)
-        index._ws_ready = True
-        return ids
-
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(steps)]
     hist = hip.new_hist(h, dev)
 
-    def step_stepwise(e=None):
-        # the separate entry points, with a dense ADC score array
+    def step(e=None):
         lut = hip.pq_build_lut(q, index.books, 1)
+        if not stepwise:
+            ids = hip.pq_search(store, index.codes, lut, q, n_cand, topk, idx_out=index.ids,
+                                workspace=index.ws, state_ready=index._ws_ready, scan_events=e)
+            index._ws_ready = True
+            return ids
+        # the separate entry points, with a dense ADC score array
         hist.zero_()
         if e is not None:
             e[0].record()
@@ -198,30 +350,80 @@ def run_pq(args, torch, hip, dev) -> int:
     for e in ev:            # events must exist before the library records them
         e[0].record()
         e[1].record()
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for s in range(args.steps):
+    for s in range(steps):
         step(ev[s])
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = (time.perf_counter() - t0) * 1e3 / steps
     scan_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / len(ev)
     scan_bytes = h * n * m
     ach = scan_bytes / (scan_ms * 1e-3) / 1e9
-    print(json.dumps({
-        "metric": "pq_adc_search_latency_us", "value": ms * 1e3, "unit": "us", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u8 codes, fp32 tables, bf16 rerank",
-        "data": "synthetic",
-        "config": {"workload": "config4: PQ baseline, 8 kv heads x 1048576 keys, hd 128, M 32 x 256 centroids, "
-                               "ADC scan -> 4096 candidates -> exact rerank to top-k 1024"},
+    # the configuration's algorithmic bytes: codes + 4096 rerank rows + codebooks + tables, per unit
+    algo = h * (n * m + n_cand * 256 + m * 256 * 4 * 4 + m * 256 * 4)
+    return {
+        "value": ms * 1e3, "unit": "us", "ms_per_step": ms, "steps": steps, "warmup": warmup,
+        "workload": C4_DESC, "dtype": "u8 codes, fp32 tables, bf16 rerank",
+        "call_path": "dc_pq_build_lut + " + ("the stepwise entry points" if stepwise else "dc_pq_search_bf16"),
         "roofline": {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": ach / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "pq_adc_kernel<32>" if args.stepwise else "pq_prune_kernel<32>",
-                     "algorithmic_bytes_per_launch": scan_bytes, "avg_launch_us": scan_ms * 1e3},
-        "cpu_baseline": None, "setup_s": t_gen}))
-    return 0
+                     "kernel": "pq_adc_kernel<32>" if stepwise else "pq_prune_kernel<32>",
+                     "algorithmic_bytes_per_launch": scan_bytes, "avg_launch_us": scan_ms * 1e3,
+                     "timed_launches": len(ev)},
+        "step_8d_bytes": algo, "step_8d_frac": algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "setup_s": t_gen,
+    }
+
+
+def cpu_baseline(torch, work: DecodeWorkload, target_s: float = 12.0) -> dict:
+    """The C restatement of the reference's exact-scan path (oracle/cpu_ref.c), timed on this
+    box's host cores on a bounded sample of the same workload.  One thread per (batch, kv-head)
+    unit, as rayon's fan-out over units does (lib.rs:387-401), with as many units in flight as
+    the box gives cores to one GPU.  The sample rotates over several layers' K/V so that no pass
+    finds its keys in the host's last-level cache."""
+    import numpy as np
+    from oracle import cpu_ref
+    cfg = work.cfg
+    hkv, hq, hd, n, b, L = cfg["hkv"], cfg["hq"], cfg["hd"], cfg["ctx"], cfg["batch"], cfg["layers"]
+    grp = hq // hkv
+    cores = os.cpu_count() or 1
+    share = min(cores, 16)                      # a GPU box gives one GPU's share of the host: 16 cores
+    nb = max(1, min(b, share // hkv))           # batch elements per pass
+    units = nb * hkv
+    threads = min(units, share)
+    n_buf = min(L, 4)                           # distinct layers to rotate over (4 x 0.5 GB of keys)
+
+    def host(t):
+        return t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+    bufs = []
+    for l in range(n_buf):
+        k, v, q, nk, nv = work.layers[l]
+        bufs.append((host(q[:nb]).reshape(units, grp, hd), host(k[:nb]).reshape(units, n, hd),
+                     host(v[:nb]).reshape(units, n, hd), host(nk[:nb]).reshape(units, hd),
+                     host(nv[:nb]).reshape(units, hd)))
+    cpu_ref.lib()
+    reps, total = 0, 0.0
+    while total < target_s and reps < 20000:
+        q0, k0, v0, nk0, nv0 = bufs[reps % n_buf]
+        t0 = time.perf_counter()
+        cpu_ref.decode_layer(q0, k0, v0, cfg["budget"], cfg["sink"], cfg["recent"], n_ctx=n,
+                             new_k_u16=nk0, new_v_u16=nv0, n_threads=threads, want_ids=False)
+        total += time.perf_counter() - t0
+        reps += 1
+    per_pass = total / reps
+    units_total = L * b * hkv
+    pass_bytes = units * n * hd * 2
+    return {
+        "value": per_pass * (units_total / units) * 1e6, "unit": "us", "cores": threads, "kind": "port",
+        "sample": (f"oracle/cpu_ref.c decode_layer (scan + heap select + gather + attention) on {units} units "
+                   f"({nb} batch element(s) of one layer, {n} rows each), {threads} threads, rotating over "
+                   f"{n_buf} layers' K/V ({n_buf * pass_bytes / 1e9:.1f} GB of keys); mean of {reps} passes = "
+                   f"{per_pass * 1e3:.2f} ms ({pass_bytes / per_pass / 1e9:.0f} GB/s of key bytes); scaled x"
+                   f"{units_total // units} to the full step ({L} layers x batch {b}); host reports {cores} cpus"),
+    }
 
 
 def main() -> int:
@@ -229,43 +431,33 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS) + ["c4"])
+    ap.add_argument("--config", default="all", choices=["all", "c2", "c3", "c4", "c5"],
+                    help="all (default): configuration 3 as the headline, both scan routes, with "
+                         "configurations 2, 4 and 5 beside it; or one configuration alone")
+    ap.add_argument("--scan", default=None, choices=["sketch", "bf16", "dense"],
+                    help="one configuration alone: sketch (default; scan the 8-bit sketch of the keys and "
+                         "rescore the surviving rows exactly from the bf16 keys), bf16 (stream the bf16 keys) "
+                         "or dense (materialise fp32 scores: dc_score_bf16 + dc_topk_select)")
     ap.add_argument("--mode", default="ref_dist", choices=["ref_dist", "ip"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--split", action="store_true",
-                    help="issue the scan, select and attention as separate C calls with an event between "
-                         "each (per-stage breakdown) instead of one dc_decode_layer call per layer")
     ap.add_argument("--event-stride", type=int, default=4,
-                    help="one-call path: time the scan kernel in place on every N-th layer")
-    ap.add_argument("--streams", type=int, default=1,
-                    help="pipeline the batch as this many independent micro-batches, one HIP stream each "
-                         "(the units of a layer are independent, so one micro-batch's select/attention "
-                         "overlaps the other's scan)")
+                    help="time the scan kernel in place on every N-th layer")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the steps, run a plain elementwise kernel that reads 1 GiB and writes "
                          "1 GiB three times (a known-size reference for FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--dense", action="store_true",
-                    help="materialise the fp32 scores (dc_score_bf16 + dc_topk_select) instead of the "
-                         "streaming score + select")
     ap.add_argument("--stepwise", action="store_true",
                     help="config c4 only: the PQ search through the separate entry points (dense ADC "
                          "score array) instead of dc_pq_search_bf16")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one decode step (all layers) in a HIP graph and time its replays; "
-                         "reported as graph_step_us next to the eager figure")
-    ap.add_argument("--scan", default=None, choices=["sketch", "bf16"],
-                    help="sketch (default): scan the 8-bit sketch of the keys and rescore the surviving "
-                         "rows exactly from the bf16 keys (same ids, half the bytes); bf16: stream the "
-                         "bf16 keys themselves")
+                         "reported as graph_step_us (always done for configuration 2)")
     args = ap.parse_args()
-    other_path = args.dense or args.split or args.streams != 1
-    if args.scan == "sketch" and other_path:
-        print("bench.py: --scan sketch goes with the default one-call path only", file=sys.stderr)
-        return 2
-    args.sketch = (args.scan or ("bf16" if other_path else "sketch")) == "sketch"
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
               "use --gpus 1", file=sys.stderr)
+        return 2
+    if args.config == "all" and args.scan is not None:
+        print("bench.py: --scan goes with a single --config", file=sys.stderr)
         return 2
 
     import torch
@@ -276,120 +468,8 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.config == "c4":
-        return run_pq(args, torch, hip, dev)
-    cfg = CONFIGS[args.config]
-    cfg_id = {"c2": 2, "c3": 3, "c5": 5}[args.config]
     mode = hip.MODE_REF_DIST if args.mode == "ref_dist" else hip.MODE_IP
-    L, b, hq, hkv, hd, n = cfg["layers"], cfg["batch"], cfg["hq"], cfg["hkv"], cfg["hd"], cfg["ctx"]
-    grp = hq // hkv
-    n_units = b * hkv
-    sink, recent, budget = cfg["sink"], cfg["recent"], cfg["budget"]
-    lo, hi = sink, n - recent
-    region = hi - lo
-    k_eff = min(budget, region)
-    attended = k_eff + sink + recent + 1
-
-    t_gen = time.perf_counter()
-    # One allocation holds every layer's keys and one every layer's values, as the KV
-    # store of diffcache_amd.DiffCache does: scans of a single large allocation run
-    # about 3 % faster on MI355X than scans of per-layer allocations.
-    vslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
-    kslab = torch.empty((L, b, hkv, n, hd), dtype=torch.bfloat16, device=dev)
-    layers = [make_layer(torch, cfg, l, cfg_id, dev, kslab[l], vslab[l]) for l in range(L)]
-    sketches = None
-    if args.sketch:
-        # the sketch of the retrieval region of every layer (prefill-time work, untimed)
-        cslab = torch.empty((L, b, hkv, n, hd), dtype=torch.uint8, device=dev)
-        sketches = [hip.Sketch(kslab[l], codes=cslab[l]).build(kslab[l], lo, hi - lo) for l in range(L)]
-    torch.cuda.synchronize()
-    t_gen = time.perf_counter() - t_gen
-
-    if args.streams < 1 or b % args.streams != 0:
-        print("bench.py: --streams must divide the batch size", file=sys.stderr)
-        return 2
-    args.fused = not args.split
-
-    class Pipe:
-        """One micro-batch: its slice of every layer's tensors, its buffers, its stream."""
-
-        def __init__(self, b0, b1):
-            self.nb = b1 - b0
-            self.n_units = self.nb * hkv
-            self.layers = [(k[b0:b1], v[b0:b1], q[b0:b1], nk[b0:b1], nv[b0:b1]) for (k, v, q, nk, nv) in layers]
-            nu = self.n_units
-            self.scores = torch.empty((nu, region), dtype=torch.float32, device=dev) if args.dense else None
-            self.idx = torch.empty((nu, budget), dtype=torch.int32, device=dev)
-            self.out = torch.empty((self.nb, hq, hd), dtype=torch.bfloat16, device=dev)
-            self.hist = hip.new_hist(nu, dev)
-            self.ws_topk = hip.alloc_workspace(hip.lib.dc_topk_workspace_bytes(nu, region, budget), dev)
-            self.ws_attn = hip.alloc_workspace(hip.lib.dc_attn_workspace_bytes(nu, grp, hd, attended), dev)
-            self.ws_layer = hip.alloc_workspace(hip.layer_workspace_bytes(nu, region, budget, grp, hd, attended), dev)
-            self.ws_sel = hip.alloc_workspace(hip.score_select_workspace_bytes(nu, region, budget), dev)
-            self.stream = torch.cuda.Stream(device=dev)     # default priority
-            self.clean = False
-
-        def layer(self, l, ev=None, wait_for=None):
-            k, v, q, nk, nv = self.layers[l]
-            nu = self.n_units
-            if wait_for is not None:
-                # scans of different micro-batches take turns: this layer call starts once the
-                # other micro-batch's scan has finished, so its select/attention overlap our scan
-                torch.cuda.current_stream().wait_event(wait_for)
-            if args.fused:
-                hip.decode_layer(q, k, v, sink, hi, recent, budget, self.scores, self.idx, self.out,
-                                 self.ws_layer, nk, nv, mode=mode, order=hip.ORDER_ANY,
-                                 select_state_ready=self.clean and not args.dense,
-                                 scan_events=None if ev is None or l % stride else
-                                 (ev[4 * l], ev[4 * l + 1]),
-                                 sketch=None if sketches is None else sketches[l])
-                self.clean = True
-                return
-            if args.dense:
-                self.hist.zero_()
-            elif not self.clean:
-                hip.select_state_init(nu, region, budget, self.ws_sel)
-                self.clean = True   # dc_sparse_select(reinit) keeps it so from here on
-            if ev is not None:
-                ev[4 * l + 0].record()
-            if args.dense:
-                hip.score(k, q, lo, region, mode, q_group=grp, scores=self.scores, hist=self.hist)
-            else:
-                hip.score_prune(k, q, lo, region, budget, self.ws_sel, mode, q_group=grp)
-            if ev is not None:
-                ev[4 * l + 1].record()
-            if args.dense:
-                hip.topk_select(self.scores, budget, mode, hip.ORDER_ANY, hist=self.hist, idx_out=self.idx,
-                                workspace=self.ws_topk)
-            else:
-                hip.sparse_select(self.idx, nu, region, budget, self.ws_sel, mode, hip.ORDER_ANY, reinit=True)
-            if ev is not None:
-                ev[4 * l + 2].record()
-            hip.gather_attn(q, k, v, self.idx, k_eff, lo, sink, hi, recent, nk, nv, out=self.out,
-                            workspace=self.ws_attn)
-            if ev is not None:
-                ev[4 * l + 3].record()
-
-    per = b // args.streams
-    pipes = [Pipe(i * per, (i + 1) * per) for i in range(args.streams)]
-
-    def new_events(count):
-        return [torch.cuda.Event(enable_timing=True) for _ in range(count)]
-
-    stride = 1 if args.streams > 1 else args.event_stride
-
-    def step(evs):
-        """One decode step: every layer in order; the micro-batches are independent of
-        each other and each runs its layers in order on its own stream.  With several
-        streams the scans are chained through their end events so that only one scan
-        streams from HBM at a time."""
-        prev_scan_end = None
-        for l in range(L):
-            for pi, pipe in enumerate(pipes):
-                with torch.cuda.stream(pipe.stream):
-                    pipe.layer(l, evs[pi], wait_for=prev_scan_end if args.streams > 1 else None)
-                if args.streams > 1:
-                    prev_scan_end = evs[pi][4 * l + 1]
+    steps, warmup = args.steps, args.warmup
 
     if args.pmc_calibration:
         ca = torch.ones((256 << 20,), dtype=torch.float32, device=dev)      # 1 GiB
@@ -399,151 +479,64 @@ def main() -> int:
         torch.cuda.synchronize()
         del ca, cb
 
-    events = [[new_events(4 * L) for _ in pipes] for _ in range(args.steps + 1)]
-    # torch creates the native event on first record; the C side needs the handle
-    for per_step in events:
-        for pi, evs in enumerate(per_step):
-            for e in evs:
-                e.record(pipes[pi].stream)
-    torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step(events[-1])
-    torch.cuda.synchronize()
-    events = events[:-1]
-    # one more event after every step on the first micro-batch's stream: the spread of the
-    # step times (with several streams the boundaries are only approximate)
-    marks = new_events(args.steps + 1)
-    for e in marks:
-        e.record(pipes[0].stream)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    marks[0].record(pipes[0].stream)
-    for s in range(args.steps):
-        step(events[s])
-        marks[s + 1].record(pipes[0].stream)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(args.steps))
+    head = {"metric": "decode_step_retrieval_sparse_attn_latency_us", "n_gpus": 1, "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
 
-    def pct(p):
-        return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
+    def line(res: dict, extra_config: dict) -> dict:
+        """The contract's keys first, then everything the measurement returned."""
+        out = dict(head)
+        out.update({"value": res["value"], "unit": res["unit"], "steps": res["steps"], "warmup": res["warmup"],
+                    "ms_per_step": res["ms_per_step"]})
+        out["config"] = dict({"workload": res["workload"], "call_path": res["call_path"]}, **extra_config)
+        for k, v in res.items():
+            if k not in ("value", "unit", "steps", "warmup", "ms_per_step", "workload", "call_path"):
+                out[k] = v
+        return out
 
-    # Small configurations fit in the 256 MB Infinity Cache, so the loop above measures a
-    # warm cache.  Cold: a 1 GiB buffer is overwritten before every step (untimed) and each
-    # step is timed on its own.
-    cold_step_us = None
-    if n_units * L * region * hd * 2 < (512 << 20) and args.streams == 1:
-        flush = torch.empty((1 << 30,), dtype=torch.uint8, device=dev)
-        c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        cold = []
-        for s_i in range(min(args.steps, 30)):
-            with torch.cuda.stream(pipes[0].stream):
-                flush.fill_(s_i & 0xff)
-                c0.record()
-            step(events[s_i])
-            with torch.cuda.stream(pipes[0].stream):
-                c1.record()
-            torch.cuda.synchronize()
-            cold.append(c0.elapsed_time(c1) * 1e3)
-        cold.sort()
-        cold_step_us = cold[len(cold) // 2]
-        del flush
+    if args.config == "c4":
+        res = measure_pq(torch, hip, dev, steps, warmup, args.stepwise)
+        out = line(res, {})
+        out["metric"] = "pq_adc_search_latency_us"
+        out["cpu_baseline"] = None
+        print(json.dumps(out))
+        return 0
 
-    graph_step_us = None
-    if args.graph and args.streams == 1 and args.fused:
-        # every call of the step only enqueues kernels on the stream, so the whole step can be
-        # captured; the select state is already "left ready" by the eager steps above
-        cap_stream = pipes[0].stream
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=cap_stream):
-            for l in range(L):
-                pipes[0].layer(l, None)
-        torch.cuda.synchronize()
-        for _ in range(max(args.warmup, 1)):
-            graph.replay()
-        torch.cuda.synchronize()
-        tg = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        graph_step_us = (time.perf_counter() - tg) * 1e6 / args.steps
+    if args.config != "all":
+        scan = args.scan or "sketch"
+        work = DecodeWorkload(torch, hip, args.config, dev, sketch=scan == "sketch")
+        res = work.measure(scan, mode, steps, warmup, args.event_stride, graph=args.graph or args.config == "c2",
+                           cold=args.config == "c2")
+        out = line(res, {"key_mode": args.mode})
+        out["setup_s"] = work.setup_s
+        out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(torch, work)
+        print(json.dumps(out))
+        return 0
 
-    # per-kernel durations from the events of the timed region
-    stage_us = None
-    score_ms = None
-    flat = [e for per_step in events for e in per_step]
-    if args.fused:
-        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(0, L, stride)]
-        score_ms = sum(sc) / len(sc)
-        stage_us = {"score": score_ms * 1e3, "timed_launches": len(sc)}
-    else:
-        sc = [e[4 * l].elapsed_time(e[4 * l + 1]) for e in flat for l in range(L)]
-        se = [e[4 * l + 1].elapsed_time(e[4 * l + 2]) for e in flat for l in range(L)]
-        at = [e[4 * l + 2].elapsed_time(e[4 * l + 3]) for e in flat for l in range(L)]
-        score_ms = sum(sc) / len(sc)
-        stage_us = {"score": score_ms * 1e3, "select": sum(se) / len(se) * 1e3,
-                    "attn": sum(at) / len(at) * 1e3, "timed_launches": len(sc)}
-
-    unit_bytes = algorithmic_bytes_per_unit(region, k_eff + sink + recent, grp, hd)
-    step_bytes = unit_bytes * n_units * L
-    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
-    # what the chosen path must move: the sketch scan reads hd bytes per key, not 2*hd
-    step_path_bytes = step_bytes - (n_units * L * region * hd if args.sketch else 0)
-    # bytes one scan launch has to stream: the bf16 K rows, or their one-byte-per-element sketch
-    score_bytes = (n_units // args.streams) * region * hd * (1 if args.sketch else 2)
-    roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
-                "traffic": None,
-                "kernel": "sketch_prune_kernel<128>" if args.sketch else
-                          "score_kernel<128>" if args.dense else "score_prune_kernel<128>",
-                "algorithmic_bytes_per_launch": score_bytes}
-    if args.config == "c3" and args.streams == 1 and not args.dense and args.mode == "ref_dist":
-        roofline["traffic"] = SCAN_TRAFFIC_BYTES_C3["sketch" if args.sketch else "bf16"]
-    if score_ms is not None:
-        ach = score_bytes / (score_ms * 1e-3) / 1e9
-        roofline.update(achieved=ach, frac=ach / HBM_PEAK_GBPS, avg_launch_us=score_ms * 1e3)
-
-    result = {
-        "metric": "decode_step_retrieval_sparse_attn_latency_us",
-        "value": ms_per_step * 1e3,
-        "unit": "us",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": cfg["desc"], "key_mode": args.mode, "streams": args.streams,
-                   "call_path": ("dc_decode_layer" + (" (dense scores)" if args.dense else
-                                                      " (sketch scan + exact rescoring)" if args.sketch else "")
-                                 if args.fused else
-                                 "dc_score_bf16/dc_topk_select/dc_gather_attn_bf16" if args.dense else
-                                 "dc_select_state_init/dc_score_prune_bf16/dc_sparse_select/dc_gather_attn_bf16")},
-        # bytes of the reference's exact algorithm per step (every bf16 key once + the gathered
-        # K/V rows + q in/out) over the measured time.  With the sketch scan the path streams
-        # one byte per key element instead of two, so this rate can exceed the HBM peak; the
-        # bytes this call path has to move are in step_path_bytes.
-        "step_hbm_gbps": step_gbps,
-        "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
-        "step_algorithmic_bytes": step_bytes,
-        "step_path_bytes": step_path_bytes,
-        "step_path_gbps": step_path_bytes / (ms_per_step * 1e-3) / 1e9,
-        "keys_scored_per_s": n_units * L * region / (ms_per_step * 1e-3),
-        "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
-        "graph_step_us": graph_step_us,
-        "cold_cache_step_us_median": cold_step_us,
-        "stage_us_per_layer": stage_us,
-        "roofline": roofline,
-        "setup_s": t_gen,
-    }
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, cfg, layers)
-    else:
-        result["cpu_baseline"] = None
-    print(json.dumps(result))
+    # ---- the default run: configuration 3 as the headline, the rest beside it -------------------
+    c3 = CONFIGS["c3"]
+    slabs = Slabs(torch, dev, c3["layers"] * c3["batch"] * c3["hkv"] * c3["ctx"] * c3["hd"], True)
+    work = DecodeWorkload(torch, hip, "c3", dev, slabs)
+    res = work.measure("sketch", mode, steps, warmup, args.event_stride)
+    out = line(res, {"key_mode": args.mode})
+    out["setup_s"] = work.setup_s
+    out["routes"] = {"bf16": work.measure("bf16", mode, steps, max(2, warmup // 2), args.event_stride)}
+    cpu = None if args.no_cpu else cpu_baseline(torch, work)
+    del work
+    configs = {}
+    w5 = DecodeWorkload(torch, hip, "c5", dev, slabs)
+    configs["c5"] = w5.measure("sketch", mode, steps, warmup, args.event_stride)
+    configs["c5"]["routes"] = {"bf16": w5.measure("bf16", mode, steps, max(2, warmup // 2), args.event_stride)}
+    del w5
+    w2 = DecodeWorkload(torch, hip, "c2", dev)
+    n2 = max(steps, 200)                        # one layer per step: more steps for a stable mean
+    configs["c2"] = w2.measure("sketch", mode, n2, max(warmup, 20), 1, graph=True, cold=True)
+    configs["c2"]["routes"] = {"bf16": w2.measure("bf16", mode, n2, max(warmup, 20), 1, graph=True, cold=True)}
+    del w2
+    store4 = slabs.k[:8 * (1 << 20) * 128].view(1, 8, 1 << 20, 128)
+    configs["c4"] = measure_pq(torch, hip, dev, max(steps, 100), max(warmup, 10), False, store4)
+    out["configs"] = configs
+    out["cpu_baseline"] = cpu
+    print(json.dumps(out))
     return 0
 
 
