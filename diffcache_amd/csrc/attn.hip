@@ -14,208 +14,21 @@
 // through their log-sum-exp.  (Merging in the last block to arrive was tried:
 // the device-scope fence it needs costs far more than a second launch here.)
 // Bound by HBM: 2 * HD*2 bytes per row.
-#include "dc_common.h"
-#include <math.h>
+#include "dc_attn.h"
 #include <mutex>
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
-// rows a lane group takes per block: 8 while the GQA group is small, 4 when the per-head
-// registers (queries, logits, accumulators) leave less room
-__host__ __device__ constexpr int rows_per_group(int group) { return group <= 4 ? 8 : 4; }
-constexpr uint32_t kNewToken = 0xffffffffu;
-
-struct AttnPlan {
-    int rows_per_split;
-    int n_splits;
-};
-
-AttnPlan plan_attn(int hd, int group, int n_total) {
-    AttnPlan p;
-    p.rows_per_split = (kThreads / (hd / 8)) * rows_per_group(group);
-    p.n_splits = n_total > 0 ? (n_total + p.rows_per_split - 1) / p.rows_per_split : 1;
-    return p;
-}
+constexpr int kThreads = kAttnThreads;
 
 template <int HD, int G>
-__global__ __launch_bounds__(kThreads) void gather_attn_kernel(
-    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
-    const uint32_t *__restrict__ idx, const uint16_t *__restrict__ new_k,
-    const uint16_t *__restrict__ new_v, float *__restrict__ ws_acc, float *__restrict__ ws_ml,
-    const uint32_t *__restrict__ n_idx_unit, const int32_t *__restrict__ n_recent_dev, int n_h, int n_idx,
-    int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent, int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
-    int64_t vsr, float scale) {
-    constexpr int LPR = HD / 8;
-    constexpr int NG = kThreads / LPR;  // row groups per block
-    constexpr int R = rows_per_group(G);
-    constexpr int ROWS = NG * R;
-    __shared__ float s_red[kWaves][G];
-    __shared__ float s_l[kWaves][G];
-    __shared__ float s_acc[kWaves][G * HD];
-
-    const int unit = blockIdx.x / n_splits;
-    const int split = blockIdx.x % n_splits;
-    const int b = unit / n_h, h = unit % n_h;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int gid = tid / LPR, col = tid % LPR;
-    const int r0 = split * ROWS;
-
-    // The length of the recent window may live on the device (the role of cache_seqlens in
-    // base.py:134-142): n_recent is then its capacity, which sized the grid, and the rows
-    // beyond the actual length are masked like any position past the end of the list.
-    if (n_recent_dev) {
-        int c = *n_recent_dev;
-        c = c < 0 ? 0 : (c < n_recent ? c : n_recent);
-        n_total -= n_recent - c;
-        n_recent = c;
-    }
-
-    // only the first n_eff selected ids of the unit count when per-unit sizes are given
-    int n_eff = n_idx;
-    if (n_idx_unit) {
-        const uint32_t ne = n_idx_unit[unit];
-        n_eff = ne < (uint32_t)n_idx ? (int)ne : n_idx;
-    }
-
-    // physical rows of this group's list positions
-    uint32_t row[R];
-    bool ok[R];
-#pragma unroll
-    for (int t = 0; t < R; ++t) {
-        const int vj = r0 + t * NG + gid;
-        ok[t] = vj < n_total && (vj < n_eff || vj >= n_idx);
-        uint32_t r = 0;
-        if (ok[t]) {
-            if (vj < n_idx) r = (uint32_t)(region_lo + idx[(int64_t)unit * idx_stride + vj]);
-            else if (vj < n_idx + n_sink) r = (uint32_t)(vj - n_idx);
-            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
-            else r = kNewToken;
-        }
-        row[t] = r;
-    }
-    float qf[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const uint4 w = *reinterpret_cast<const uint4 *>(Q + ((int64_t)unit * G + g) * HD + col * 8);
-        qf[g][0] = dc_bf16_lo(w.x);
-        qf[g][1] = dc_bf16_hi(w.x);
-        qf[g][2] = dc_bf16_lo(w.y);
-        qf[g][3] = dc_bf16_hi(w.y);
-        qf[g][4] = dc_bf16_lo(w.z);
-        qf[g][5] = dc_bf16_hi(w.z);
-        qf[g][6] = dc_bf16_lo(w.w);
-        qf[g][7] = dc_bf16_hi(w.w);
-    }
-    const uint16_t *Ku = K + b * ksb + h * ksh + col * 8;
-    const uint16_t *Vu = V + b * vsb + h * vsh + col * 8;
-    const uint16_t *nk = new_k ? new_k + (int64_t)unit * HD + col * 8 : Ku;
-    const uint16_t *nv = new_v ? new_v + (int64_t)unit * HD + col * 8 : Vu;
-
-    // every K and V row of the slice is requested before any is used
-    uint4 kw[R], vw[R];
-#pragma unroll
-    for (int t = 0; t < R; ++t) {
-        const uint16_t *pk = (row[t] == kNewToken) ? nk : Ku + (int64_t)row[t] * ksr;
-        kw[t] = *reinterpret_cast<const uint4 *>(pk);
-    }
-#pragma unroll
-    for (int t = 0; t < R; ++t) {
-        const uint16_t *pv = (row[t] == kNewToken) ? nv : Vu + (int64_t)row[t] * vsr;
-        vw[t] = *reinterpret_cast<const uint4 *>(pv);
-    }
-
-    // scaled logits, in registers: x[t][g] is known to every lane of the group
-    float x[R][G];
-    float mloc[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) mloc[g] = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < R; ++t)
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float v = dc_group_sum<LPR>(dc_dot8(kw[t], qf[g], 0.f)) * scale;
-            x[t][g] = ok[t] ? v : -INFINITY;
-            mloc[g] = fmaxf(mloc[g], x[t][g]);
-        }
-    // per-head maximum over the block
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float v = mloc[g];
-#pragma unroll
-        for (int off = LPR; off < 64; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-        if (lane == 0) s_red[wave][g] = v;
-    }
-    __syncthreads();
-    float m[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float v = s_red[0][g];
-#pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) v = fmaxf(v, s_red[w2][g]);
-        m[g] = v;
-    }
-
-    // p = exp(x - m), acc[g] += p * V
-    float acc[G][8];
-    float lloc[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        lloc[g] = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-    }
-#pragma unroll
-    for (int t = 0; t < R; ++t) {
-        const float v[8] = {dc_bf16_lo(vw[t].x), dc_bf16_hi(vw[t].x), dc_bf16_lo(vw[t].y),
-                            dc_bf16_hi(vw[t].y), dc_bf16_lo(vw[t].z), dc_bf16_hi(vw[t].z),
-                            dc_bf16_lo(vw[t].w), dc_bf16_hi(vw[t].w)};
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float p = ok[t] ? __expf(x[t][g] - m[g]) : 0.f;
-            lloc[g] += p;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
-        }
-    }
-
-    // reduce over the row groups: inside the wave, then across waves
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1)
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            lloc[g] += __shfl_xor(lloc[g], off, 64);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] += __shfl_xor(acc[g][i], off, 64);
-        }
-    if (lane < LPR) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            if (col == 0) s_l[wave][g] = lloc[g];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s_acc[wave][g * HD + col * 8 + i] = acc[g][i];
-        }
-    }
-    __syncthreads();
-    const int64_t slot = (int64_t)unit * n_splits + split;
-    for (int o = tid; o < G * HD; o += kThreads) {
-        float s = s_acc[0][o];
-#pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) s += s_acc[w2][o];
-        ws_acc[slot * (G * HD) + o] = s;
-    }
-    if (tid < G) {
-        float l = s_l[0][tid];
-#pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) l += s_l[w2][tid];
-        float mm = s_red[0][tid];
-#pragma unroll
-        for (int w2 = 1; w2 < kWaves; ++w2) mm = fmaxf(mm, s_red[w2][tid]);
-        ws_ml[(slot * G + tid) * 2 + 0] = mm;
-        ws_ml[(slot * G + tid) * 2 + 1] = l;
-    }
-
+__global__ __launch_bounds__(kThreads) void gather_attn_kernel(AttnArgs a) {
+    __shared__ float s_mem[attn_shared_floats<HD, G>()];
+    AttnShared sh;
+    sh.red = s_mem;
+    sh.l = s_mem + kAttnWaves * G;
+    sh.acc = s_mem + 2 * kAttnWaves * G;
+    dc_attn_split<HD, G, false>(a, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, sh);
 }
 
 // out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block
@@ -298,38 +111,11 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
     if (out_v) *reinterpret_cast<uint4 *>(out_v + dst) = *reinterpret_cast<const uint4 *>(V + src);
 }
 
-struct AttnWs {
-    float *acc, *ml;
-    size_t bytes;
-};
-
-AttnWs carve_attn(void *base, int n_units, int group, int hd, int n_splits) {
-    AttnWs w;
-    char *p = (char *)base;
-    size_t off = 0;
-    const size_t slots = (size_t)(n_units > 0 ? n_units : 0) * (size_t)n_splits;
-    w.acc = (float *)(p + off);
-    off += dc_align_up(slots * group * hd * 4, 256);
-    w.ml = (float *)(p + off);
-    off += dc_align_up(slots * group * 2 * 4, 256);
-    w.bytes = off;
-    return w;
-}
-
 template <int HD>
-int launch_attn(int group, dim3 grid, hipStream_t st, const uint16_t *q, const uint16_t *k,
-                const uint16_t *v, const uint32_t *idx, const uint16_t *new_k,
-                const uint16_t *new_v, const AttnWs &w, const uint32_t *n_idx_unit,
-                const int32_t *n_recent_dev, int n_h, int n_idx,
-                int64_t idx_stride, int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
-                int n_total, int n_splits, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
-                int64_t vsh, int64_t vsr, float scale) {
-#define DC_ATTN_CASE(GG)                                                                           \
-    case GG:                                                                                       \
-        hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, q, k, v, idx, \
-                           new_k, new_v, w.acc, w.ml, n_idx_unit, n_recent_dev, n_h, n_idx, idx_stride,        \
-                           region_lo, n_sink, recent_lo, n_recent, n_total, n_splits, ksb, ksh,    \
-                           ksr, vsb, vsh, vsr, scale);                                             \
+int launch_attn(int group, dim3 grid, hipStream_t st, const AttnArgs &a) {
+#define DC_ATTN_CASE(GG)                                                                      \
+    case GG:                                                                                  \
+        hipLaunchKernelGGL((gather_attn_kernel<HD, GG>), grid, dim3(kThreads), 0, st, a);      \
         return 0;
     switch (group) {
         DC_ATTN_CASE(1)
@@ -394,22 +180,33 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     DC_REQUIRE((int64_t)n_units * plan.n_splits < (1ll << 31), "%s: grid too large", who);
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)((size_t)n_units * plan.n_splits));
-    int rc;
-    const uint16_t *q16 = (const uint16_t *)q, *k16 = (const uint16_t *)k, *v16 = (const uint16_t *)v;
-    const uint16_t *nk16 = (const uint16_t *)new_k, *nv16 = (const uint16_t *)new_v;
+    AttnArgs aa;
+    aa.Q = (const uint16_t *)q;
+    aa.K = (const uint16_t *)k;
+    aa.V = (const uint16_t *)v;
+    aa.idx = idx;
+    aa.new_k = (const uint16_t *)new_k;
+    aa.new_v = (const uint16_t *)new_v;
+    aa.ws_acc = w.acc;
+    aa.ws_ml = w.ml;
+    aa.n_idx_unit = n_idx_unit;
+    aa.n_recent_dev = n_recent_dev;
+    aa.n_h = n_h;
+    aa.n_idx = n_idx;
+    aa.idx_stride = idx_unit_stride;
+    aa.region_lo = region_lo;
+    aa.n_sink = n_sink;
+    aa.recent_lo = recent_lo;
+    aa.n_recent = n_recent;
+    aa.n_total = n_total;
+    aa.n_splits = plan.n_splits;
+    aa.ksb = ksb, aa.ksh = ksh, aa.ksr = ksr, aa.vsb = vsb, aa.vsh = vsh, aa.vsr = vsr;
+    aa.scale = scale;
     uint16_t *o16 = (uint16_t *)out;
-    if (hd == 64)
-        rc = launch_attn<64>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
-                             idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                             plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
-    else if (hd == 128)
-        rc = launch_attn<128>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
-                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
-    else
-        rc = launch_attn<256>(group, grid, st, q16, k16, v16, idx, nk16, nv16, w, n_idx_unit, n_recent_dev, n_h, n_idx,
-                              idx_unit_stride, region_lo, n_sink, recent_lo, n_recent, n_total,
-                              plan.n_splits, ksb, ksh, ksr, vsb, vsh, vsr, scale);
+    int rc;
+    if (hd == 64) rc = launch_attn<64>(group, grid, st, aa);
+    else if (hd == 128) rc = launch_attn<128>(group, grid, st, aa);
+    else rc = launch_attn<256>(group, grid, st, aa);
     DC_REQUIRE(rc == 0, "%s: unsupported group %d", who, group);
     DC_CHECK_LAUNCH(who);
     hipLaunchKernelGGL(merge_kernel, dim3((unsigned)(n_units * group)), dim3(hd), 0, st, w.acc, w.ml, o16,
