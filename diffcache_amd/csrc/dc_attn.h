@@ -1,6 +1,5 @@
 // Decode attention over gathered K/V rows: the per-split body and the merge of the splits,
-// shared by the stand-alone kernels (attn.hip) and by the fused tail of a decode layer
-// (tail.hip).  Replaces flash_attn_with_kvcache over the assembled buffer
+// used by the attention kernels (attn.hip).  Replaces flash_attn_with_kvcache over the assembled buffer
 // (src/diffcache/base.py:134-142, src/diffcache/kvcache/diffcache.py:196-209).
 //
 // A split is a slice of rows_per_group * NG consecutive positions of a unit's attended list

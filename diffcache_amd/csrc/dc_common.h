@@ -34,6 +34,12 @@ int dc_sort_selected(const float *scores, int64_t scores_stride, const uint32_t 
                      uint32_t *idx_out, int64_t idx_stride, unsigned long long *scratch, int n_units,
                      int k_eff, int mode, int order, hipStream_t st, int n_rows);
 
+// fused.hip: argument checks, state initialisation and the scan kernel of the sketch route
+int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, const float *scale,
+                          const float *resid, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb,
+                          int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group, int budget,
+                          int mode, int state_ready, void *workspace, size_t workspace_bytes,
+                          void *ev_scan_begin, void *ev_scan_end, void *stream);
 static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 

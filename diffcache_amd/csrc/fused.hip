@@ -30,37 +30,10 @@
 // select_finish_kernel picks the k best of that list.
 #include "dc_common.h"
 #include "dc_select.h"
+#include "dc_fused.h"
 #include "dc_pq.h"
 
 namespace {
-
-constexpr int kThreads = 256;
-constexpr int kRowsPerBlockStep = 256;
-constexpr int kBigSteps = 8;       // 2048 rows per large block
-constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
-constexpr int kStage = kBigSteps * kRowsPerBlockStep;
-constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
-constexpr int kSharedPollUnits = 8;   // sketch scan: up to this many units, one wave per block polls
-constexpr int kPqThreads = 512;    // PQ scan: threads per block = keys per step
-constexpr int kPqBigSteps = 8;     // PQ scan: 4096 keys per large block
-constexpr int kBinsPerThread = DC_HIST_BINS / kThreads;  // bins a thread owns when a block scans a histogram
-static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kThreads == DC_HIST_BINS, "bin split");
-
-// tb_run is polled by every wave of the scan while surv_cnt takes returning
-// atomics; they sit in separate 128-byte lines because polling a line that is
-// being updated atomically serialises both at the memory side.
-struct UnitState {
-    uint32_t tb_run;    // running threshold bucket (only decreases)
-    uint32_t pad0[31];
-    uint32_t surv_cnt;  // survivors appended so far
-    uint32_t win_cnt;   // certain members written to idx_out (select phase)
-    uint32_t cand_cnt;  // candidates of the threshold bucket (select phase)
-    uint32_t c_less;    // keys in buckets better than the threshold bucket
-    uint32_t margin;    // sketch scan only: float bits of the score margin of the unit
-    uint32_t pad1[27];
-};
-static_assert(sizeof(UnitState) == 256, "UnitState is two 128-byte lines");
-static_assert(kRadixBins * 4 >= kFinalThreads * 8, "lh doubles as the packed candidate list");
 
 __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -74,10 +47,6 @@ __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units)
         state[i].c_less = 0;
         state[i].margin = 0;
     }
-}
-
-__device__ __forceinline__ uint32_t load_relaxed(const uint32_t *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // A block's copy of its unit's running threshold bucket, in LDS.  The poll of the unit's
@@ -552,48 +521,6 @@ __global__ __launch_bounds__(kPqThreads) void pq_prune_kernel(
                                    refresh, (uint32_t)k_eff);
 }
 
-// Exact threshold bucket of a unit from its complete histogram: the bucket that
-// holds the k-th best key, and how many keys sit in better buckets.  Called by
-// all kThreads threads; the result is uniform.  `wtot`, `sres`: LDS scratch.
-__device__ __forceinline__ void unit_threshold(const uint32_t *__restrict__ hu, uint32_t kk,
-                                               uint32_t *wtot, uint32_t *sres, uint32_t &tb,
-                                               uint32_t &c_less) {
-    const int tid = threadIdx.x;
-    if (tid == 0) {
-        sres[0] = DC_HIST_BINS;
-        sres[1] = 0;
-    }
-    uint32_t bins[kBinsPerThread];
-    uint32_t sum = 0;
-#pragma unroll
-    for (int i = 0; i < kBinsPerThread / 4; ++i) {
-        const uint4 t = reinterpret_cast<const uint4 *>(hu)[tid * (kBinsPerThread / 4) + i];
-        bins[4 * i + 0] = t.x;
-        bins[4 * i + 1] = t.y;
-        bins[4 * i + 2] = t.z;
-        bins[4 * i + 3] = t.w;
-        sum += t.x + t.y + t.z + t.w;
-    }
-    uint32_t total;
-    const uint32_t excl = block_excl_scan<kThreads>(sum, wtot, &total);
-    if (excl < kk && kk <= excl + sum) {
-        uint32_t run = excl;
-        bool done = false;
-#pragma unroll
-        for (int i = 0; i < kBinsPerThread; ++i) {
-            if (!done && run + bins[i] >= kk) {
-                sres[0] = tid * kBinsPerThread + i;
-                sres[1] = run;
-                done = true;
-            }
-            run += bins[i];
-        }
-    }
-    __syncthreads();
-    tb = sres[0];
-    c_less = sres[1];
-}
-
 // Several blocks per unit split the unit's survivor list: rows in buckets better
 // than the threshold bucket are certain members and go straight to idx_out, rows
 // in the threshold bucket become candidates.  Each block reserves its output
@@ -920,45 +847,6 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
                      ko ? ko + c_less : nullptr);
 }
 
-struct FusedWs {
-    uint32_t *hist;
-    UnitState *state;
-    uint2 *surv;
-    uint32_t *cand_key, *cand_idx, *sel_keys;
-    unsigned long long *sort_scratch;
-    size_t bytes;
-};
-
-int fused_pow2(int x) {
-    int p = 1;
-    while (p < x) p <<= 1;
-    return p;
-}
-
-FusedWs carve_fused(void *base, int n_units, int n_rows, int k) {
-    FusedWs w;
-    char *p = (char *)base;
-    size_t off = 0;
-    const size_t nu = n_units > 0 ? n_units : 0, nr = n_rows > 0 ? n_rows : 0;
-    const int keff = k < n_rows ? k : n_rows;
-    w.hist = (uint32_t *)(p + off);
-    off += dc_align_up(nu * DC_HIST_BINS * 4, 256);
-    w.state = (UnitState *)(p + off);
-    off += dc_align_up(nu * sizeof(UnitState), 256);
-    w.surv = (uint2 *)(p + off);
-    off += dc_align_up(nu * nr * 8, 256);
-    w.cand_key = (uint32_t *)(p + off);
-    off += dc_align_up(nu * nr * 4, 256);
-    w.cand_idx = (uint32_t *)(p + off);
-    off += dc_align_up(nu * nr * 4, 256);
-    w.sel_keys = (uint32_t *)(p + off);
-    off += dc_align_up(nu * (size_t)(keff > 0 ? keff : 0) * 4, 256);
-    w.sort_scratch = (unsigned long long *)(p + off);
-    if (keff > 4096) off += dc_align_up(nu * (size_t)fused_pow2(keff) * 8, 256);
-    w.bytes = off;
-    return w;
-}
-
 }  // namespace
 
 extern "C" size_t dc_score_select_workspace_bytes(int n_units, int n_rows, int k) {
@@ -1131,19 +1019,17 @@ extern "C" int dc_sketch_select_state_init(int n_units, int n_rows, int budget, 
     return dc_select_state_init(n_units, n_rows, budget, workspace, workspace_bytes, stream);
 }
 
-extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, const float *scale,
-                                           const float *resid, const void *q, uint32_t *idx_out,
-                                           int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
-                                           int64_t sb, int64_t sh, int64_t sr, int64_t cb, int64_t ch,
-                                           int64_t cr, int q_group, int budget, int mode, int order,
-                                           int state_ready, void *workspace, size_t workspace_bytes,
-                                           void *ev_scan_begin, void *ev_scan_end, void *stream) {
-    const char *who = "dc_score_select_sketch_bf16";
-    DC_REQUIRE(k && codes && scale && resid && q && idx_out, "%s: null pointer", who);
+// Checks, state initialisation and the scan kernel of the sketch route; what follows the scan
+// (exact pass, selection) is enqueued by the caller.
+int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, const float *scale,
+                          const float *resid, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb,
+                          int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group, int budget,
+                          int mode, int state_ready, void *workspace, size_t workspace_bytes,
+                          void *ev_scan_begin, void *ev_scan_end, void *stream) {
+    DC_REQUIRE(k && codes && scale && resid && q, "%s: null pointer", who);
     DC_REQUIRE(q_group >= 1, "%s: bad q_group", who);
     DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d not in {64,128,256}", who, hd);
     DC_REQUIRE(mode == DC_MODE_IP || mode == DC_MODE_REF_DIST, "%s: bad mode %d", who, mode);
-    DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "%s: bad order %d", who, order);
     DC_REQUIRE(dc_aligned16(k) && dc_aligned16(codes) && dc_aligned16(scale) && dc_aligned16(resid),
                "%s: k, codes, scale and resid must be 16-byte aligned", who);
     DC_REQUIRE(sb % 8 == 0 && sh % 8 == 0 && sr % 8 == 0 && sr >= hd,
@@ -1154,7 +1040,6 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
     int rc = plan_fused(who, n_b, n_h, n_rows, budget, &p);
     if (rc) return rc;
     if (p.n_units == 0 || p.k_eff == 0) return DC_OK;
-    DC_REQUIRE(idx_unit_stride >= p.k_eff, "%s: idx_unit_stride < min(budget, n_rows)", who);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "%s: workspace must be non-null and 256-byte aligned", who);
     const FusedWs w = carve_fused(workspace, p.n_units, n_rows, budget);
@@ -1182,6 +1067,30 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
 #undef DC_LAUNCH_SK
     DC_CHECK_LAUNCH(who);
     if (ev_scan_end) (void)hipEventRecord((hipEvent_t)ev_scan_end, st);
+    return DC_OK;
+}
+
+extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, const float *scale,
+                                           const float *resid, const void *q, uint32_t *idx_out,
+                                           int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                                           int64_t sb, int64_t sh, int64_t sr, int64_t cb, int64_t ch,
+                                           int64_t cr, int q_group, int budget, int mode, int order,
+                                           int state_ready, void *workspace, size_t workspace_bytes,
+                                           void *ev_scan_begin, void *ev_scan_end, void *stream) {
+    const char *who = "dc_score_select_sketch_bf16";
+    DC_REQUIRE(idx_out, "%s: null pointer", who);
+    DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "%s: bad order %d", who, order);
+    int rc = dc_sketch_scan_launch(who, k, codes, scale, resid, q, n_b, n_h, n_rows, hd, sb, sh, sr, cb, ch, cr,
+                                   q_group, budget, mode, state_ready, workspace, workspace_bytes,
+                                   ev_scan_begin, ev_scan_end, stream);
+    if (rc) return rc;
+    FusedPlan p;
+    rc = plan_fused(who, n_b, n_h, n_rows, budget, &p);
+    if (rc) return rc;
+    if (p.n_units == 0 || p.k_eff == 0) return DC_OK;
+    DC_REQUIRE(idx_unit_stride >= p.k_eff, "%s: idx_unit_stride < min(budget, n_rows)", who);
+    const FusedWs w = carve_fused(workspace, p.n_units, n_rows, budget);
+    hipStream_t st = (hipStream_t)stream;
     // blocks per unit of the exact pass: one per 2048 rows of context, grid near 2048 blocks
     int nblk = (n_rows + 2047) / 2048;
     const int cap = p.n_units >= 2048 ? 1 : 2048 / p.n_units;
