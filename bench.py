@@ -174,18 +174,20 @@ class DecodeWorkload:
         self.stream = torch.cuda.Stream(device=dev)     # default priority
         self.clean = False
 
-    def layer(self, l: int, scan: str, mode: int, ev=None):
+    def layer(self, l: int, scan: str, mode: int, ev=None, route_only: bool = False):
         """One dc_decode_layer call.  scan: "sketch", "bf16" or "dense" (fp32 scores +
         dc_topk_select).  ev: an event pair recorded around the scan kernel."""
         hip, cfg = self.hip, self.cfg
         k, v, q, nk, nv = self.layers[l]
         if scan == "dense" and self.scores is None:
             self.scores = self.torch.empty((self.n_units, self.region), dtype=self.torch.float32, device=self.dev)
-        hip.decode_layer(q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
-                         self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv,
-                         mode=mode, order=hip.ORDER_ANY,
-                         select_state_ready=self.clean and scan != "dense", scan_events=ev,
-                         sketch=self.sketches[l] if scan == "sketch" else None)
+        args = (q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
+                self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv)
+        kw = dict(mode=mode, order=hip.ORDER_ANY, select_state_ready=self.clean and scan != "dense",
+                  scan_events=ev, sketch=self.sketches[l] if scan == "sketch" else None)
+        if route_only:
+            return hip.decode_layer_route(*args, **kw)
+        hip.decode_layer(*args, **kw)
         self.clean = scan != "dense"
 
     def measure(self, scan: str, mode: int, steps: int, warmup: int, event_stride: int = 4,
@@ -280,12 +282,22 @@ class DecodeWorkload:
         rows_bytes_8d = nu * self.region * hd * 2             # one launch, every bf16 key row once
         scan_bytes = rows_bytes_8d // 2 if scan == "sketch" else rows_bytes_8d + \
             (nu * self.region * 4 if scan == "dense" else 0)
+        kernel = {"sketch": "sketch_prune_kernel<128>", "bf16": "score_prune_kernel<128>",
+                  "dense": "score_kernel<128>"}[scan]
+        call_path = "dc_decode_layer" + {"sketch": " (sketch scan + exact rescoring)", "bf16": "",
+                                         "dense": " (dense scores)"}[scan]
+        if self.layer(0, scan, mode, route_only=True) == self.hip.ROUTE_ONE_KERNEL:
+            # short context: the layer is one kernel that reads the bf16 keys (with or without a
+            # sketch) and the event pair brackets all of it
+            kernel = "small_layer_kernel<%d, %d>" % (hd, self.grp)
+            call_path = "dc_decode_layer (short context: one kernel)"
+            path_bytes = step_bytes
+            scan_bytes = unit_bytes * nu
         ach = scan_bytes / (scan_ms * 1e-3) / 1e9
         roofline = {
             "bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBPS,
             "traffic": None,
-            "kernel": {"sketch": "sketch_prune_kernel<128>", "bf16": "score_prune_kernel<128>",
-                       "dense": "score_kernel<128>"}[scan],
+            "kernel": kernel,
             "algorithmic_bytes_per_launch": scan_bytes, "avg_launch_us": scan_ms * 1e3,
             "timed_launches": len(sc),
             # the same launch priced at the reference algorithm's bytes (two per key element)
@@ -300,8 +312,7 @@ class DecodeWorkload:
         return {
             "value": ms_per_step * 1e3, "unit": "us", "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
             "workload": cfg["desc"], "scan": scan,
-            "call_path": "dc_decode_layer" + {"sketch": " (sketch scan + exact rescoring)", "bf16": "",
-                                              "dense": " (dense scores)"}[scan],
+            "call_path": call_path,
             "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
             "roofline": roofline,
             # bytes this route must move per step over the step time: the step-level HBM fraction

@@ -29,6 +29,7 @@ SYMBOLS = (
     "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
     "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_gather_attn_static_bf16", "dc_append_kv_bf16",
     "dc_step_advance", "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
+    "dc_decode_layer_status", "dc_set_wait_limit", "dc_decode_layer_route",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
     "dc_sparse_select", "dc_score_select_bf16",
@@ -87,6 +88,9 @@ def _load() -> C.CDLL:
         "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
         "dc_layer_workspace_bytes": (sz, [i, i, i, i, i, i]),
         "dc_decode_layer": (i, [C.POINTER(LayerArgs), p]),
+        "dc_decode_layer_status": (i, [C.POINTER(LayerArgs), p]),
+        "dc_set_wait_limit": (None, [i]),
+        "dc_decode_layer_route": (i, [C.POINTER(LayerArgs)]),
         "dc_pq_build_lut": (i, [p, p, p, i, i, i, i, p]),
         "dc_pq_adc_scan": (i, [p, p, p, p, i, i, i, i64, p]),
         "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
@@ -502,20 +506,10 @@ def layer_workspace_bytes(n_units: int, n_region: int, budget: int, group: int, 
     return int(lib.dc_layer_workspace_bytes(n_units, n_region, budget, group, hd, n_attended))
 
 
-def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, n_sink: int,
-                 recent_lo: int, n_recent: int, budget: int, scores: Optional[torch.Tensor],
-                 idx_out: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor,
-                 new_k: Optional[torch.Tensor] = None, new_v: Optional[torch.Tensor] = None,
-                 lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
-                 order: int = ORDER_ANY, scale: Optional[float] = None,
-                 select_state_ready: bool = False,
-                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
-                 sketch: Optional["Sketch"] = None,
-                 n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """score -> select -> attend for one layer, enqueued on the current stream.
-    ``n_recent_dev``: the suffix length as a device-side int32 (``n_recent`` = capacity).
-    ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
-    ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result)."""
+def _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
+                new_k=None, new_v=None, lse=None, mode=MODE_REF_DIST, order=ORDER_ANY, scale=None,
+                select_state_ready=False, scan_events=None, sketch=None, n_recent_dev=None) -> "LayerArgs":
+    """struct dc_layer_args from tensors (the arguments of decode_layer), with their checks."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
         raise DiffCacheError("K and V stores must share their strides")
@@ -557,8 +551,48 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
         a.sketch_resid = _dev(sketch.resid, "resid")
         a.sketch_batch_stride, a.sketch_head_stride, a.sketch_row_stride = c.stride(0), c.stride(1), c.stride(2)
     a.n_recent_dev = _counter(n_recent_dev)
+    a._keep = (q, store_k, store_v, new_k, new_v, out, lse, scores, idx_out, workspace, sketch, n_recent_dev)
+    return a
+
+
+def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, n_sink: int,
+                 recent_lo: int, n_recent: int, budget: int, scores: Optional[torch.Tensor],
+                 idx_out: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor,
+                 new_k: Optional[torch.Tensor] = None, new_v: Optional[torch.Tensor] = None,
+                 lse: Optional[torch.Tensor] = None, mode: int = MODE_REF_DIST,
+                 order: int = ORDER_ANY, scale: Optional[float] = None,
+                 select_state_ready: bool = False,
+                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
+                 sketch: Optional["Sketch"] = None,
+                 n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """score -> select -> attend for one layer, enqueued on the current stream.
+    ``n_recent_dev``: the suffix length as a device-side int32 (``n_recent`` = capacity).
+    ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
+    ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result)."""
+    a = _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
+                    new_k, new_v, lse, mode, order, scale, select_state_ready, scan_events, sketch, n_recent_dev)
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
+
+
+ROUTE_ATTEND_ONLY, ROUTE_DENSE, ROUTE_STREAM, ROUTE_SKETCH, ROUTE_ONE_KERNEL = range(5)
+
+
+def decode_layer_route(*args, **kwargs) -> int:
+    """Which kernels a decode_layer call with these arguments runs: a ROUTE_* value."""
+    a = _layer_args(*args, **kwargs)
+    rc = lib.dc_decode_layer_route(C.byref(a))
+    if rc < 0:
+        _check(rc)
+    return rc
+
+
+def decode_layer_status(*args, **kwargs) -> None:
+    """Waits for the current stream and raises if a kernel of the last decode_layer calls on this
+    workspace gave up a bounded wait between its blocks (dc_decode_layer_status).  Arguments as
+    in the decode_layer call that it checks."""
+    a = _layer_args(*args, **kwargs)
+    _check(lib.dc_decode_layer_status(C.byref(a), _stream()))
 
 
 # ---- PQ baseline ----

@@ -1,5 +1,7 @@
 // Error plumbing, version, and the fused per-layer call chain of the C ABI.
 #include "dc_common.h"
+#include <vector>
+#include "dc_fused.h"
 #include <stdarg.h>
 #include <string.h>
 
@@ -47,7 +49,11 @@ LayerWs carve_layer(void *base, int n_units, int n_region, int budget, int group
     }
     off += w.topk_bytes;
     w.attn = p + off;
-    w.attn_bytes = dc_align_up(dc_attn_workspace_bytes(n_units, group, hd, n_attended), 256);
+    {   // split partials of the attention kernels, or of the one-kernel route for short contexts
+        size_t a = dc_attn_workspace_bytes(n_units, group, hd, n_attended);
+        size_t b = dc_small_workspace_bytes(n_units, n_region, group, hd);
+        w.attn_bytes = dc_align_up(a > b ? a : b, 256);
+    }
     off += w.attn_bytes;
     w.bytes = off;
     return w;
@@ -87,6 +93,21 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     int rc;
     const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
+    if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY &&
+        dc_small_supported(n_units, region, k_eff, a->group, a->hd)) {
+        // short context: the whole layer in one kernel whose blocks are all resident (ids in no
+        // particular order); reads the bf16 keys, with or without a sketch
+        if (!a->select_state_ready) {
+            rc = dc_select_state_init(n_units, region, a->budget, w.topk, w.topk_bytes, stream);
+            if (rc) return rc;
+            rc = dc_small_state_init(n_units, region, a->budget, w.topk, stream);
+            if (rc) return rc;
+        }
+        if (a->ev_scan_begin) (void)hipEventRecord((hipEvent_t)a->ev_scan_begin, st);
+        rc = dc_small_launch(a, region, k_eff, w.topk, w.attn, w.attn_bytes, stream);
+        if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
+        return rc;
+    }
     if (k_eff > 0 && !a->scores && a->sketch_codes) {
         // streaming select over the 8-bit sketch, exact rescoring of the kept rows
         DC_REQUIRE(a->sketch_scale && a->sketch_resid, "dc_decode_layer: sketch_scale / sketch_resid missing");
@@ -133,4 +154,44 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
                              a->kv_row_stride, a->kv_batch_stride, a->kv_head_stride,
                              a->kv_row_stride, a->scale, w.attn, w.attn_bytes, stream);
     return rc;
+}
+
+extern "C" int dc_decode_layer_route(const dc_layer_args *a) {
+    DC_REQUIRE(a, "dc_decode_layer_route: null args");
+    const int n_units = a->n_b * a->n_h;
+    const int64_t region64 = a->recent_lo - a->n_sink;
+    DC_REQUIRE(n_units >= 0 && region64 >= 0 && region64 < (1ll << 31), "dc_decode_layer_route: bad sizes");
+    const int region = (int)region64;
+    const int k_eff = a->budget < region ? a->budget : region;
+    if (n_units == 0 || k_eff <= 0) return DC_ROUTE_ATTEND_ONLY;
+    if (a->scores) return DC_ROUTE_DENSE;
+    if (a->order == DC_ORDER_ANY && dc_small_supported(n_units, region, k_eff, a->group, a->hd)) return DC_ROUTE_ONE_KERNEL;
+    return a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;
+}
+
+extern "C" int dc_decode_layer_status(const dc_layer_args *a, void *stream) {
+    DC_REQUIRE(a && a->workspace, "dc_decode_layer_status: null args or workspace");
+    const int n_units = a->n_b * a->n_h;
+    if (n_units <= 0) return DC_OK;
+    const int region = (int)(a->recent_lo - a->n_sink);
+    const int k_eff = a->budget < region ? a->budget : region;
+    const LayerWs w = carve_layer(a->workspace, n_units, region, a->budget, a->group, a->hd,
+                                  k_eff + a->n_sink + a->n_recent + (a->new_k ? 1 : 0));
+    DC_REQUIRE(a->workspace_bytes >= w.bytes, "dc_decode_layer_status: workspace too small");
+    const FusedWs f = carve_fused(w.topk, n_units, region, a->budget);
+    std::vector<uint32_t> err((size_t)n_units, 0u);
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipMemcpy2DAsync(err.data(), sizeof(uint32_t), &f.state[0].sync_err, sizeof(UnitState),
+                                    sizeof(uint32_t), (size_t)n_units, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) {
+        dc_set_error("dc_decode_layer_status: %s", hipGetErrorString(e));
+        return DC_ELAUNCH;
+    }
+    for (int u = 0; u < n_units; ++u)
+        if (err[(size_t)u]) {
+            dc_set_error("dc_decode_layer_status: unit %d gave up a bounded wait between its blocks", u);
+            return DC_EDEVICE;
+        }
+    return DC_OK;
 }

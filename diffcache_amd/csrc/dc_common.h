@@ -40,6 +40,13 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
                           int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group, int budget,
                           int mode, int state_ready, void *workspace, size_t workspace_bytes,
                           void *ev_scan_begin, void *ev_scan_end, void *stream);
+// small.hip: a whole decode layer in one kernel, for short contexts
+bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd);
+size_t dc_small_workspace_bytes(int n_units, int region, int group, int hd);
+int dc_small_state_init(int n_units, int region, int budget, void *sel_ws, void *stream);
+int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws, void *attn_ws,
+                    size_t attn_ws_bytes, void *stream);
+
 static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 

@@ -22,13 +22,18 @@ static_assert(kBinsPerThread % 4 == 0 && kBinsPerThread * kThreads == DC_HIST_BI
 // being updated atomically serialises both at the memory side.
 struct UnitState {
     uint32_t tb_run;    // running threshold bucket (only decreases)
-    uint32_t pad0[31];
+    uint32_t sync_cnt;  // one-kernel route (small.hip): arrivals of the unit's blocks at its barriers; zero between launches
+    uint32_t pad0[30];
     uint32_t surv_cnt;  // survivors appended so far
     uint32_t win_cnt;   // certain members written to idx_out (select phase)
     uint32_t cand_cnt;  // candidates of the threshold bucket (select phase)
     uint32_t c_less;    // keys in buckets better than the threshold bucket
     uint32_t margin;    // sketch scan only: float bits of the score margin of the unit
-    uint32_t pad1[27];
+    // the one-kernel route for short contexts (small.hip)
+    uint32_t sync_err;  // a bounded wait ran out (never expected)
+    uint32_t cut_key;   // the cutoff (key, id) when a unit's candidates are too many to rank in LDS
+    uint32_t cut_id;
+    uint32_t pad1[24];
 };
 static_assert(sizeof(UnitState) == 256, "UnitState is two 128-byte lines");
 static_assert(kRadixBins * 4 >= kFinalThreads * 8, "lh doubles as the packed candidate list");

@@ -46,6 +46,10 @@ __global__ void init_state_kernel(uint32_t *hist, UnitState *state, int n_units)
         state[i].cand_cnt = 0;
         state[i].c_less = 0;
         state[i].margin = 0;
+        state[i].sync_cnt = 0;
+        state[i].sync_err = 0;
+        state[i].cut_key = 0;
+        state[i].cut_id = 0;
     }
 }
 

@@ -143,6 +143,7 @@ class DiffCache:
         # by the stand-alone select calls, so each route keeps its own "left ready" flag and
         # clears the other's.
         self._ws_ready = False        # a decode_attention call has left its select state ready
+        self._ws_order = None         # ... for calls of this id order
         self._hook_ws_ready = False   # a decode_query_kvcache call (sketch route) has
         self._attn_out: Optional[torch.Tensor] = None
         # k-check (nsw.rs:198-296): with use_k_check, decode_attention attends only to the
@@ -372,9 +373,11 @@ class DiffCache:
             # attended: [selected | prefix | the window's rows before this token | this token]
             hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
                              self.kvbuf_suffix_maxlen, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
-                             nk, nv, mode=self.mode, order=order, select_state_ready=self._ws_ready,
+                             nk, nv, mode=self.mode, order=order,
+                             select_state_ready=self._ws_ready and self._ws_order == order,
                              sketch=self.sketch[layer_idx], n_recent_dev=self.step_state)
             self._ws_ready = True
+            self._ws_order = order      # the state is left ready for a call of the same order only
             self._hook_ws_ready = False
         if layer_idx == self.num_layers - 1:
             hip.step_advance(self.step_state, 1, self.kvbuf_suffix_maxlen)

@@ -46,6 +46,7 @@ extern "C" {
 #define DC_EINVAL (-22)
 #define DC_ENOMEM (-12)   /* workspace too small */
 #define DC_ELAUNCH (-5)   /* hipLaunchKernel failed */
+#define DC_EDEVICE (-6)   /* a kernel gave up a bounded wait: the outputs of that call are not valid */
 
 #define DC_HIST_BINS 1024 /* histogram bins per unit used by the select */
 
@@ -327,9 +328,10 @@ typedef struct dc_layer_args {
     float scale;          /* softmax scale, 1/sqrt(hd) in the reference */
     int select_state_ready; /* streaming select only (scores == NULL).  0: the workspace is
                              initialised first.  1: the caller vouches that the last call on this
-                             workspace was a dc_decode_layer with the same n_b, n_h, region length
-                             and budget and scores == NULL (with or without a sketch), which
-                             leaves the select state ready; the init kernel is skipped */
+                             workspace was a dc_decode_layer with the same n_b, n_h, group, hd,
+                             region length, budget and order and scores == NULL (with or without
+                             a sketch), which leaves the select state ready; the init kernels
+                             are skipped */
     void *ev_scan_begin;  /* optional hipEvent_t pair recorded on `stream` right before and */
     void *ev_scan_end;    /* right after the scan kernel (for timing it in place), or NULL */
     const uint8_t *sketch_codes; /* NULL, or the sketch of the K store (row 0 = store row 0): the
@@ -345,6 +347,33 @@ typedef struct dc_layer_args {
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,
                                 int n_rows_attended);
 int dc_decode_layer(const dc_layer_args *args, void *stream);
+/*
+ * Short contexts.  With scores == NULL, order == DC_ORDER_ANY and at most 640 Ki region rows
+ * over all units, dc_decode_layer runs the layer as ONE kernel whose blocks are all resident
+ * and hand their phases over through the workspace (same results; the event pair then brackets
+ * that kernel).  Its waits between blocks are bounded; dc_decode_layer_status waits for
+ * `stream` and returns DC_EDEVICE if a wait of the last calls on this workspace ran out (never
+ * observed; the outputs would be invalid), DC_OK otherwise.  `args` as in the call it checks.
+ * No counterpart in the reference, whose layers run on the CPU pool (lib.rs:352-369).
+ */
+int dc_decode_layer_status(const dc_layer_args *args, void *stream);
+/*
+ * Which kernels a dc_decode_layer call with these arguments runs (pointers are not followed):
+ * a DC_ROUTE_* value, or a negative DC_E* code.
+ */
+#define DC_ROUTE_ATTEND_ONLY 0 /* nothing to select (empty region or budget 0) */
+#define DC_ROUTE_DENSE 1       /* fp32 scores materialised: dc_score_bf16 + dc_topk_select */
+#define DC_ROUTE_STREAM 2      /* dc_score_prune_bf16 + dc_sparse_select */
+#define DC_ROUTE_SKETCH 3      /* dc_score_select_sketch_bf16 */
+#define DC_ROUTE_ONE_KERNEL 4  /* short context: the whole layer in one kernel */
+int dc_decode_layer_route(const dc_layer_args *args);
+/*
+ * For tests of that error path: the number of polls after which a block of the one-kernel
+ * route gives up a wait (0: the default, about a second).  With a tiny limit the kernel still
+ * runs to its end, its outputs are not valid, dc_decode_layer_status reports DC_EDEVICE and the
+ * next call on the workspace needs select_state_ready == 0.  Process-wide.
+ */
+void dc_set_wait_limit(int polls);
 
 /*
  * PQ asymmetric-distance baseline.  The reference's PQ baseline directory

@@ -1,0 +1,169 @@
+"""The one-kernel route of dc_decode_layer for short contexts (csrc/small.hip).
+
+dc_decode_layer takes it when no dense scores are asked for, the ids may come in any order and
+every block of the launch fits on the chip at once.  Checked against the oracle like the other
+routes: ids bit-exact against ``oracle.topk_select`` of the GPU's dense scores (the kept set of
+search_bruteforce, diffcache_cpu/src/nsw.rs:592-630, ties to the lower id), attention within
+2e-3 of the float64 softmax over the oracle's row set (src/diffcache/base.py:134-142).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+hip = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global hip
+    from diffcache_amd import _hip
+    hip = _hip
+    yield
+
+
+def to_dev_bf16(u16):
+    return torch.from_numpy(u16.view(np.int16).copy()).view(torch.bfloat16).to(DEV)
+
+
+def to_np_u16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def bf16_close(got_f32, want_f64):
+    tol = np.maximum(2e-3, np.abs(want_f64) * 2.0 ** -8)
+    return bool(np.all(np.abs(got_f32 - want_f64) <= tol))
+
+
+def run_case(k, v, q, nk, nv, n_ctx, budget, p, s, mode, reps=2, n_recent_dev=None, recent_cap=None, ws=None):
+    """k, v (b, hkv, n_max, hd) u16; q (b, hq, hd); nk, nv (b, hkv, hd) or None.  Calls
+    dc_decode_layer (no scores, ORDER_ANY) `reps` times on one workspace and checks every call."""
+    b, hkv, n_max, hd = k.shape
+    hq = q.shape[1]
+    g = hq // hkv
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, p, s)
+    region = hi - lo
+    k_eff = min(budget, region)
+    n_units = b * hkv
+    kd, vd, qd = to_dev_bf16(k), to_dev_bf16(v), to_dev_bf16(q)
+    nkd = None if nk is None else to_dev_bf16(nk)
+    nvd = None if nv is None else to_dev_bf16(nv)
+    cap = s_len if recent_cap is None else recent_cap
+    if ws is None:
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(n_units, region, budget, g, hd,
+                                                           k_eff + p_len + cap + 1), DEV)
+    dense = hip.score(kd, qd, lo, region, mode, q_group=g).cpu().numpy() if region > 0 else None
+    lse = torch.empty((b, hq), dtype=torch.float32, device=DEV)
+    for rep in range(reps):
+        idx = torch.full((n_units, max(budget, 1)), -1, dtype=torch.int32, device=DEV)
+        out = torch.full((b, hq, hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        args = (qd, kd, vd, p_len, hi, cap, budget, None, idx, out, ws, nkd, nvd)
+        kw = dict(lse=lse, mode=mode, order=hip.ORDER_ANY, select_state_ready=rep > 0, n_recent_dev=n_recent_dev)
+        hip.decode_layer(*args, **kw)
+        hip.decode_layer_status(*args, **kw)        # waits for the stream; no bounded wait ran out
+        ids = idx.cpu().numpy()[:, :k_eff].astype(np.int64)
+        got = orc.bf16_to_f32(to_np_u16(out))
+        got_lse = lse.cpu().numpy()
+        for u in range(n_units):
+            bi, h = divmod(u, hkv)
+            want = orc.topk_select(dense[u], k_eff, mode).astype(np.int64) if k_eff else np.zeros(0, np.int64)
+            assert np.array_equal(np.sort(ids[u]), np.sort(want)), (rep, u)
+            rows = np.concatenate([want + lo, np.arange(p_len), np.arange(hi, hi + s_len)]).astype(np.int64)
+            o, l = orc.sparse_attention(q[bi, h * g:(h + 1) * g], k[bi, h][rows], v[bi, h][rows],
+                                        None if nk is None else nk[bi, h], None if nv is None else nv[bi, h])
+            assert bf16_close(got[bi, h * g:(h + 1) * g], o), (rep, u)
+            assert np.allclose(got_lse[bi, h * g:(h + 1) * g], l, rtol=1e-4, atol=1e-4), (rep, u)
+    return ws
+
+
+def rand_bf16(rng, *shape, scale=1.0):
+    return orc.f32_to_bf16((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("hd,hq,hkv", [(128, 8, 2), (64, 7, 7), (256, 16, 2), (128, 14, 2)])
+def test_small_context_layer_matches_oracle(mode, hd, hq, hkv):
+    rng = np.random.default_rng(300 + hd + hq)
+    b, n_ctx = 2, 5000
+    k, v = rand_bf16(rng, b, hkv, n_ctx + 3, hd), rand_bf16(rng, b, hkv, n_ctx + 3, hd)
+    q = rand_bf16(rng, b, hq, hd)
+    nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+    print(f"small context hd={hd} hq={hq} hkv={hkv} mode={mode}", flush=True)
+    run_case(k, v, q, nk, nv, n_ctx, 300, 4, 64, mode)
+
+
+def test_small_context_edge_sizes_share_one_workspace():
+    """Regions of 1 row, fewer rows than the budget, no current token, no sinks; consecutive calls of
+    different sizes each initialise their own state."""
+    rng = np.random.default_rng(301)
+    b, hq, hkv, hd = 1, 8, 2, 128
+    for n_ctx, budget, p, s, tok in [(70, 64, 4, 64, True), (69, 64, 4, 64, True), (300, 512, 4, 64, False),
+                                     (4000, 128, 0, 0, True), (2500, 1, 2, 3, True), (9000, 4096, 4, 64, True)]:
+        print(f"small context n_ctx={n_ctx} budget={budget} p={p} s={s} tok={tok}", flush=True)
+        k, v = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd)
+        q = rand_bf16(rng, b, hq, hd)
+        nk = rand_bf16(rng, b, hkv, hd) if tok else None
+        nv = rand_bf16(rng, b, hkv, hd) if tok else None
+        run_case(k, v, q, nk, nv, n_ctx, budget, p, s, orc.MODE_REF_DIST)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_small_context_ties(mode):
+    """Integer-valued keys: scores tie in large groups, the boundary goes to the lower ids.  A zero
+    query makes every row tie (more candidates than a block ranks in LDS: the radix-select path)."""
+    rng = np.random.default_rng(302 + mode)
+    b, hq, hkv, hd, n_ctx = 1, 12, 3, 128, 20000
+    k = orc.f32_to_bf16(rng.integers(-2, 3, (b, hkv, n_ctx, hd)).astype(np.float32))
+    v = rand_bf16(rng, b, hkv, n_ctx, hd)
+    q = orc.f32_to_bf16(rng.integers(-1, 2, (b, hq, hd)).astype(np.float32))
+    q[0, 8:12] = 0                                      # unit 2: everything ties, lowest ids win
+    k[0, 1, 5000:15000] = k[0, 1, 4999]                 # unit 1: ten thousand identical rows
+    nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+    run_case(k, v, q, nk, nv, n_ctx, 1500, 4, 64, mode)
+
+
+def test_small_context_benchmark_shape_with_a_device_side_window():
+    """Benchmark configuration 2 (8 units x 32700 rows, k 1024, outlier channels); the recent
+    window's length is read from the device and grows between the calls."""
+    rng = np.random.default_rng(303)
+    b, hq, hkv, hd, n0, cap = 1, 32, 8, 128, 32768, 72
+    scale = np.exp(rng.standard_normal((1, hkv, 1, hd))).astype(np.float32)
+    k = orc.f32_to_bf16(rng.standard_normal((b, hkv, n0 + 8, hd)).astype(np.float32) * scale)
+    v = rand_bf16(rng, b, hkv, n0 + 8, hd)
+    q = rand_bf16(rng, b, hq, hd)
+    nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+    counter = torch.zeros((1,), dtype=torch.int32, device=DEV)
+    ws = None
+    for step in range(3):
+        # the region stays [4, n0 - 64); the window holds 64 + step rows of its capacity of 72
+        counter.fill_(64 + step)
+        n_ctx = n0 + step
+        # oracle side: prefix 4, suffix 64 + step  ->  same region; the store holds the whole window
+        ws = run_case(k, v, q, nk, nv, n_ctx, 1024, 4, 64 + step,
+                      orc.MODE_REF_DIST, reps=1, n_recent_dev=counter, recent_cap=cap, ws=ws)
+
+
+def test_small_context_bounded_wait_is_reported():
+    """With a wait limit of one poll the blocks give up their waits: the kernel still ends, the
+    status call reports it, and after a fresh initialisation the route works again."""
+    rng = np.random.default_rng(304)
+    b, hq, hkv, hd, n_ctx = 1, 8, 2, 128, 30000
+    k, v = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd)
+    q = rand_bf16(rng, b, hq, hd)
+    kd, vd, qd = to_dev_bf16(k), to_dev_bf16(v), to_dev_bf16(q)
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+    ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, 512, hq // hkv, hd, 512 + 4 + 64 + 1), DEV)
+    idx = torch.zeros((b * hkv, 512), dtype=torch.int32, device=DEV)
+    out = torch.empty((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    args = (qd, kd, vd, p_len, hi, s_len, 512, None, idx, out, ws)
+    hip.lib.dc_set_wait_limit(1)
+    try:
+        hip.decode_layer(*args, order=hip.ORDER_ANY)
+        with pytest.raises(hip.DiffCacheError, match="bounded wait"):
+            hip.decode_layer_status(*args, order=hip.ORDER_ANY)
+    finally:
+        hip.lib.dc_set_wait_limit(0)
+    run_case(k, v, q, None, None, n_ctx, 512, 4, 64, orc.MODE_REF_DIST, reps=2, ws=ws)
