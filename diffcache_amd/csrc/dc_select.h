@@ -7,6 +7,7 @@ namespace {
 constexpr int kFinalThreads = 1024;
 constexpr int kRadixBits = 11;
 constexpr int kRadixBins = 1 << kRadixBits;
+constexpr int kScanBatch = 8;  // items of a list that a thread fetches before it looks at any
 
 // inclusive scan over the lanes of a wave
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
@@ -40,6 +41,26 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, 
     return off + incl - v;
 }
 
+// f(key, id) for every entry of a (key, id) list, kScanBatch entries of a thread in flight.
+template <int NT, typename F>
+__device__ __forceinline__ void dc_for_each_pair(const uint32_t *ck, const uint32_t *ci, uint32_t n, F f) {
+    for (uint32_t i0 = threadIdx.x; i0 < n; i0 += kScanBatch * NT) {
+        uint32_t key[kScanBatch], id[kScanBatch];
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) {
+            const uint32_t i = i0 + (uint32_t)u * NT;
+            key[u] = id[u] = 0u;
+            if (i < n) {
+                key[u] = ck[i];
+                id[u] = ci[i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u)
+            if (i0 + (uint32_t)u * NT < n) f(key[u], id[u]);
+    }
+}
+
 // One radix pass of a select: among the items whose bits [31, top) equal those of
 // `prefix`, histogram bits [top-1, top-width) and find the bin that holds the
 // rem-th smallest (1-based).  Updates prefix (bin bits filled in), rem (rank inside
@@ -54,10 +75,32 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
     for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
     __syncthreads();
     const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
-    for (uint32_t i = tid; i < n; i += kFinalThreads) {
-        uint32_t v;
-        if (get(i, &v) && ((v & himask) == (prefix & himask)))
-            atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
+    // kScanBatch items of a thread are fetched before any is looked at: with one load per
+    // iteration a long list costs a memory round trip per item and thread.  A wave whose lanes
+    // all hit one bin (long runs of equal keys) adds its count once.
+    for (uint32_t i0 = tid; i0 < n; i0 += kScanBatch * kFinalThreads) {
+        uint32_t v[kScanBatch];
+        bool in[kScanBatch];
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) {
+            const uint32_t i = i0 + (uint32_t)u * kFinalThreads;
+            v[u] = 0u;
+            in[u] = i < n && get(i, &v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) {
+            const bool hit = in[u] && ((v[u] & himask) == (prefix & himask));
+            const uint32_t bin = (v[u] >> shift) & ((1u << width) - 1u);
+            const unsigned long long hits = __ballot(hit);
+            if (hits == 0ull) continue;
+            const int leader = (int)__builtin_ctzll(hits);
+            const uint32_t lead = (uint32_t)__builtin_amdgcn_readlane((int)bin, leader);
+            if (__ballot(hit && bin != lead) == 0ull) {
+                if ((tid & 63) == leader) atomicAdd(&lh[lead], (uint32_t)__popcll(hits));
+            } else if (hit) {
+                atomicAdd(&lh[bin], 1u);
+            }
+        }
     }
     __syncthreads();
     // kRadixBins == 2 * kFinalThreads: each thread owns two adjacent bins
@@ -108,6 +151,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
                                  uint32_t *sres, uint32_t *smisc, uint32_t *kout = nullptr) {
     const int tid = threadIdx.x;
     if (need == n_c) {  // the whole candidate list is selected
+#pragma unroll 4
         for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
             io[i] = ci[i];
             if (kout) kout[i] = ck[i];
@@ -122,7 +166,16 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
     __syncthreads();
     const uint32_t k0 = ck[0];
     uint32_t diff = 0;
-    for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
+    for (uint32_t i0 = tid; i0 < n_c; i0 += kScanBatch * kFinalThreads) {
+        uint32_t v[kScanBatch];
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) {
+            const uint32_t i = i0 + (uint32_t)u * kFinalThreads;
+            v[u] = i < n_c ? ck[i] : k0;
+        }
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) diff |= v[u] ^ k0;
+    }
     if (diff) atomicOr(&smisc[0], diff);
     __syncthreads();
     diff = smisc[0];
@@ -146,8 +199,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
         __syncthreads();
         const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
         const uint32_t base = need - rem;  // members from the bins below the threshold bin
-        for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
-            const uint32_t key = ck[i], id = ci[i];
+        dc_for_each_pair<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id) {
             const uint32_t hi = key & himask, ph = prefix & himask;
             if (hi < ph) {
                 const uint32_t slot = atomicAdd(&smisc[1], 1u);
@@ -159,7 +211,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
                 const uint32_t e = atomicAdd(&smisc[0], 1u);
                 if (e < (uint32_t)kFinalThreads) tie[e] = ((unsigned long long)key << 32) | id;
             }
-        }
+        });
         __syncthreads();
         const uint32_t n_t = smisc[0] < (uint32_t)kFinalThreads ? smisc[0] : (uint32_t)kFinalThreads;
         if ((uint32_t)tid < n_t) {
@@ -190,8 +242,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
         t_idx = block_radix_select(get_idx, n_c, need_eq, hbi + 1, 0u, n_eq, lh, wtot, sres, &r2, &e2);
     }
 
-    for (uint32_t i = tid; i < n_c; i += kFinalThreads) {
-        const uint32_t key = ck[i], id = ci[i];
+    dc_for_each_pair<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id) {
         if (key < t_key || (key == t_key && id <= t_idx)) {
             uint32_t slot = atomicAdd(&smisc[1], 1u);
             if (slot < need) {
@@ -199,7 +250,7 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
                 if (kout) kout[slot] = key;
             }
         }
-    }
+    });
 }
 
 }  // namespace

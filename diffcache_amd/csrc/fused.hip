@@ -28,6 +28,7 @@
 // sketch.hip) with a margin that makes its pruning safe, rescore_kernel computes
 // the exact scores of the rows that survive it and lists them as candidates, and
 // select_finish_kernel picks the k best of that list.
+#include <type_traits>
 #include "dc_common.h"
 #include "dc_select.h"
 #include "dc_fused.h"
@@ -255,6 +256,9 @@ __device__ __forceinline__ float sketch_dot16(const uint4 &c, const float (&w)[1
 // yields the bucket of A_k exactly as in score_prune_kernel, and a row is kept when
 // bucket(approx_i + margin) is not worse than the running threshold bucket,
 // margin = 2E' + Q.  The kept rows are rescored exactly by rescore_kernel.
+constexpr uint32_t kBulkKeep = 96;      // of the 128 rows of a wave's first two steps
+constexpr float kUnseenApprox = 3.0e38f;  // approximation of a row the scan did not read: better than any score
+
 template <int HD, bool SHARED_POLL>
 __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kernel(
     const uint8_t *__restrict__ C, const uint16_t *__restrict__ Q, const float *__restrict__ scale,
@@ -331,7 +335,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     __syncthreads();
 
     uint2 *wstage = stage + wave * (kBigSteps * 64);
-    uint32_t wcnt = 0;
+    uint32_t wcnt = 0, marginal = 0;
     const unsigned long long lt = (1ull << lane) - 1ull;
 
     // Double buffering: the loads of the next step are issued before the current step is
@@ -349,7 +353,9 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
             cv[j] = dc_load_stream16(Cu + r * cr);
         }
     };
-    auto work_step = [&](int step, const uint4 (&cv)[LPR]) {
+    // COUNT: also count the rows kept although their own bucket is not better than the
+    // threshold's (ties and near-ties); only the first two steps of a wave do.
+    auto work_step = [&](int step, const uint4 (&cv)[LPR], auto count) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
         float mine = 0.f;
 #pragma unroll
@@ -365,6 +371,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
         const unsigned long long mask = __ballot(keep);
         if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
         wcnt += (uint32_t)__popcll(mask);
+        if (decltype(count)::value) marginal += (uint32_t)__popcll(__ballot(keep && lb >= tb));
     };
     // steps of this wave that hold rows (wave-uniform)
     int my_steps = 0;
@@ -378,6 +385,8 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     }
     uint4 ca[LPR], cb2[LPR];
     load_step(0, ca);
+    bool bulk = false;
+    const bool had_tb = tb < (uint32_t)DC_HIST_BINS;  // the first steps are judged against a real threshold
     // The threshold poll is issued before the prefetch: loads return in order, so waiting
     // for a poll that was issued last would also wait for the whole prefetch.
     int step = 0;
@@ -386,11 +395,11 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     // polls and passes the value on through LDS.  With many units every wave polls for
     // itself, which keeps its threshold one step fresher.
     // (SHARED_POLL is a template parameter: as a run-time choice it costs registers.)
-    for (; step + 1 < my_steps; step += 2) {
+    auto two_steps = [&](auto count) {
         uint32_t tb_next = tb;
         if (!SHARED_POLL || wave == 0) tb_next = load_relaxed(&st->tb_run);
         load_step(step + 1, cb2);
-        work_step(step, ca);
+        work_step(step, ca, count);
         if (SHARED_POLL) {
             if (wave == 0 && lane == 0) lds_store_relaxed(&s_tb, tb_next);
             tb = lds_load_relaxed(&s_tb);
@@ -399,15 +408,37 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
         }
         if (!SHARED_POLL || wave == 0) tb_next = load_relaxed(&st->tb_run);
         load_step(step + 2, ca);
-        work_step(step + 1, cb2);
+        work_step(step + 1, cb2, count);
         if (SHARED_POLL) {
             if (wave == 0 && lane == 0) lds_store_relaxed(&s_tb, tb_next);
             tb = lds_load_relaxed(&s_tb);
         } else {
             tb = tb_next;
         }
+        step += 2;
+    };
+    if (my_steps >= 2) {
+        two_steps(std::true_type{});
+        // Degenerate data (rows that nearly all tie with the k-th best: the sketch prunes nothing):
+        // a wave that kept three quarters of the rows of its first two steps without any of them
+        // being better than the threshold stops reading codes and keeps the rest of its rows unseen.
+        // An unseen row carries the best possible approximation, so the exact rescoring takes it
+        // in any case, and it is left out of the histogram, which only loosens the threshold: the
+        // selected ids are the same, the scan costs a quarter.
+        bulk = had_tb && marginal >= kBulkKeep;
     }
-    if (step < my_steps) work_step(step, ca);  // an odd last step; its rows are already on the way
+    while (!bulk && step + 1 < my_steps) two_steps(std::false_type{});
+    if (bulk) {
+        for (; step < my_steps; ++step) {
+            const int64_t myrow = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64 + lane;
+            const bool keep = myrow < n_rows;
+            const unsigned long long mask = __ballot(keep);
+            if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(kUnseenApprox));
+            wcnt += (uint32_t)__popcll(mask);
+        }
+    } else if (step < my_steps) {
+        work_step(step, ca, std::false_type{});  // an odd last step; its rows are already on the way
+    }
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
                        surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);

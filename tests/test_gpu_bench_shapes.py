@@ -51,9 +51,12 @@ def build_layer(cfg_name: str, cfg_id: int, layer: int = 0):
     return cfg, k, v, q, nk, nv
 
 
-def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units):
-    """The benchmark's layer call on its three routes against the oracle."""
+def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units, mutate=None):
+    """The benchmark's layer call on its three routes against the oracle.  mutate(k, q): changes
+    the keys in place before the sketch is built."""
     cfg, k, v, q, nk, nv = build_layer(cfg_name, cfg_id)
+    if mutate is not None:
+        mutate(k, q)
     b, hq, hkv, hd, n = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["hd"], cfg["ctx"]
     sink, recent, budget = cfg["sink"], cfg["recent"], cfg["budget"]
     grp, n_units = hq // hkv, b * hkv
@@ -131,6 +134,19 @@ def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units):
     print(f"{cfg_name}: worst attention error = {worst_abs:.2e} absolute; {worst_small:.2e} where |out| < 0.5 "
           f"(literal bar 2e-3); {worst_ulp:.2f} bf16 ulps of the output (0.5 = correctly rounded)", flush=True)
     return ids["dense"], sc
+
+
+def test_config3_layer_with_long_runs_of_equal_keys():
+    """The data that defeat every pruning scan, at the headline shape: in the even units 70000
+    consecutive rows equal one vector that scores best (the k-th best lies inside the run, the
+    lowest ids of the run win); in the odd units every row is equal.  The sketch scan stops
+    reading codes inside such runs and hands the rows to the exact pass unseen."""
+    def mutate(k, q):
+        b, hkv, n, hd = k.shape
+        qm = q.view(b, hkv, -1, hd).float().mean(2)
+        k[:, 0::2, 30000:100000] = (3.0 * torch.sign(qm[:, 0::2])).to(torch.bfloat16).unsqueeze(2)
+        k[:, 1::2] = k[:, 1::2, 77:78].clone()
+    check_layer("c3", 3, attn_units=[0, 1, 62, 63], score_units=[], mutate=mutate)
 
 
 def test_config3_one_full_layer_all_routes():

@@ -354,7 +354,8 @@ def test_sketch_select_matches_dense_path(mode, hd, n_rows, budget):
 
 
 @pytest.mark.parametrize("law", ["heavy_tail", "tiny", "huge", "sparse", "one_hot_query", "constant_rows",
-                                 "sorted_scores", "negative_scores"])
+                                 "sorted_scores", "negative_scores", "plateau_at_the_threshold",
+                                 "plateau_above_the_threshold"])
 def test_sketch_select_is_exact_on_awkward_data(law):
     """Whatever the data do to the sketch's fit, the ids are those of the exact scan."""
     rng = np.random.default_rng(sum(map(ord, law)))
@@ -384,6 +385,10 @@ def test_sketch_select_is_exact_on_awkward_data(law):
     elif law == "negative_scores":     # every score negative
         kf = -np.abs(kf)
         qf = np.abs(qf)
+    elif law.startswith("plateau"):    # a long run of equal rows that score best: the scan stops
+        lo_r, hi_r = (6000, 18000) if law == "plateau_at_the_threshold" else (11000, 11500)
+        kf[:, :, lo_r:hi_r] = 3.0 * np.sign(qf)[:, :, None, :]     # reading codes inside it; with
+        # more equal rows than the budget the lowest ids of the run win, with fewer all of it is in
     k, q = orc.f32_to_bf16(kf), orc.f32_to_bf16(qf)
     for mode in (0, 1):
         if law in ("huge",) and mode == 1:
