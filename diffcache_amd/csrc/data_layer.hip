@@ -116,6 +116,17 @@ extern "C" int dc_data_layer_bind(dc_data_layer *dl, void *k_store, void *v_stor
 }
 
 // lib.rs:329-347: keys, vals (bsz, kv_heads, n_rows, hd) bf16, host or device memory
+// true for a pointer the runtime does not know: ordinary (pageable) host memory
+static bool pageable_host(const void *p) {
+    hipPointerAttribute_t attr;
+    const hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // older runtimes report an unknown pointer as an error
+        return true;
+    }
+    return attr.type == hipMemoryTypeUnregistered;
+}
+
 extern "C" int dc_data_layer_prefill(dc_data_layer *dl, const void *keys, const void *vals, int64_t n_rows,
                                      void *stream) {
     const char *who = "dc_data_layer_prefill";
@@ -132,6 +143,10 @@ extern "C" int dc_data_layer_prefill(dc_data_layer *dl, const void *keys, const 
         hipError_t e = hipMemcpy2DAsync(dl->k, (size_t)sh * 2, keys, width, width, height, hipMemcpyDefault, st);
         if (e == hipSuccess)
             e = hipMemcpy2DAsync(dl->v, (size_t)sh * 2, vals, width, width, height, hipMemcpyDefault, st);
+        // A source in pageable host memory (not allocated by HIP) cannot be read by the copy
+        // engine behind the caller's back: the runtime stages it, and the caller may free or
+        // reuse it as soon as this call returns only if the copy is complete by then.
+        if (e == hipSuccess && (pageable_host(keys) || pageable_host(vals))) e = hipStreamSynchronize(st);
         if (e != hipSuccess) {
             dc_set_error("%s: copy failed: %s", who, hipGetErrorString(e));
             return DC_ELAUNCH;

@@ -51,7 +51,8 @@ def init_metrics() -> None:
 
 def metrics() -> Dict[str, int]:
     """Counters named as in the reference: ``<name>_num_searches``,
-    ``<name>_total_query_latency`` (microseconds of host time spent in query)."""
+    ``<name>_total_query_latency`` (microseconds from the start of a query to the end of its
+    search on the device: with metrics on, a query with device outputs waits for its stream)."""
     return dict(_metrics)
 
 
@@ -231,7 +232,12 @@ class DiffCacheHIP:
                     dst[:, :, :ef_eff, :] = host
                 else:
                     dst.view(torch.int16)[:, :, :ef_eff, :] = torch.from_numpy(host.view(np.int16))
-        _count(f"{self.name}_total_query_latency", (time.perf_counter() - t0) * 1e6)
+        if _metrics_on:
+            # the reference's counter is the time of the search itself (lib.rs:373-404 runs it to the
+            # end before it returns); with device outputs the call above only enqueued it
+            if dev_out:
+                torch.cuda.current_stream(self.device).synchronize()
+            _count(f"{self.name}_total_query_latency", (time.perf_counter() - t0) * 1e6)
 
     def query_streaming(self, cuda_stream: int, out_keys_gpu: int, out_vals_gpu: int,
                         queries: ArrayLike, ef: int) -> None:

@@ -84,7 +84,14 @@ class DiffCache:
         device: str = "cuda",
         key_sketch: bool = True,
         use_k_check: bool = False,
+        hook_order: int = hip.ORDER_BEST,
     ) -> None:
+        # hook_order: order of the ids that decode_query_kvcache selects, hence of the rows that
+        # decode_post_query_operation gathers into kbuf/vbuf.  ORDER_BEST is the reference's
+        # (best first, nsw.rs:592-630); attention over the buffer does not depend on the order, so
+        # a caller that only attends may pass hip.ORDER_ANY and save the sort.
+        hip.require(hook_order in (hip.ORDER_ANY, hip.ORDER_BEST, hip.ORDER_INDEX), "bad hook_order")
+        self.hook_order = hook_order
         self.num_layers = num_layers
         self.batch_size = batch_size
         self.max_length = max_length
@@ -308,12 +315,12 @@ class DiffCache:
             ws = self._ensure_workspace()
             if self.key_sketch:
                 hip.score_select_sketch(self.kstore[layer_idx], self.sketch[layer_idx], self.qbuf, lo, hi - lo,
-                                        retrieval_len, self.mode, hip.ORDER_BEST, idx_out=self.idx[layer_idx],
+                                        retrieval_len, self.mode, self.hook_order, idx_out=self.idx[layer_idx],
                                         workspace=ws, state_ready=self._hook_ws_ready)
                 self._hook_ws_ready = True
             else:
                 hip.score_select(self.kstore[layer_idx], self.qbuf, lo, hi - lo, retrieval_len, self.mode,
-                                 hip.ORDER_BEST, idx_out=self.idx[layer_idx], workspace=ws)
+                                 self.hook_order, idx_out=self.idx[layer_idx], workspace=ws)
                 self._hook_ws_ready = False   # the one-shot call does not leave the state initialised
             self._ws_ready = False
         hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,

@@ -438,16 +438,20 @@ int dc_pq_search_bf16(const void *k, const uint8_t *codes, const float *lut, con
  *            scale and resid (0 without the sketch), idx_bytes, workspace_bytes; max_ef =
  *            the largest ef a query will ask for.
  *   bind     hands the buffers over (16-byte aligned, the workspace 256-byte aligned).
- *   prefill  lib.rs:329-347: keys, vals (bsz, kv_heads, n_rows, hd) bf16 in host or device
- *            memory replace the contents; n_rows <= max_ctx_len.
+ *   prefill  lib.rs:329-347: keys, vals (bsz, kv_heads, n_rows, hd) bf16 replace the
+ *            contents; n_rows <= max_ctx_len.  From device memory or pinned host memory
+ *            (hipHostMalloc) the copy is enqueued and the source must stay unchanged until
+ *            `stream` has passed it; from ordinary pageable host memory (a numpy array, a
+ *            malloc'd block) the call waits for `stream` and returns with the copy done, so
+ *            the source may be reused at once -- at the price of a synchronisation.
  *   insert   lib.rs:352-369: keys, vals (bsz, kv_heads, hd) bf16 in device memory, one
  *            token per unit, appended at ctx_len; an error when the store is full.
  *   query    lib.rs:373-404 with nsw.rs:592-630: queries (bsz, kv_heads, hd) bf16; the
  *            min(ef, ctx_len) best K and V rows of every unit, best first, ties to the
  *            lower id, into out_keys / out_vals (bsz, kv_heads, out_rows, hd) in device
  *            memory; *n_out (may be NULL) = rows written per unit.
- * prefill, insert and query only enqueue work on `stream`; calls on one handle must not
- * overlap.  destroy frees the handle, never the buffers.
+ * prefill (from device or pinned memory), insert and query only enqueue work on `stream`;
+ * calls on one handle must not overlap.  destroy frees the handle, never the buffers.
  */
 typedef struct dc_data_layer dc_data_layer;
 int dc_data_layer_create(dc_data_layer **out, int bsz, int kv_heads, int hd, int64_t max_ctx_len,

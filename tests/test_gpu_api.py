@@ -232,6 +232,35 @@ def test_diffcache_hooks_assemble_the_reference_buffer(seq):
     assert cache.kvbuf_suffix_len == s_len + 1               # grows once per step (diffcache.py:222-223)
 
 
+@pytest.mark.parametrize("key_sketch", [True, False])
+def test_diffcache_hooks_in_any_order_hold_the_same_rows(key_sketch):
+    """hook_order=ORDER_ANY: the retrieved part of the buffer is a permutation of the reference's
+    best-first list (K and V rows permuted alike); prefix and suffix are unchanged."""
+    from diffcache_amd import _hip
+    rng = np.random.default_rng(12)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 1, 1, 2, 8, 128, 300, 16, 32, 64, 4000
+    cache = make_cache(L, b, seq + 40, hkv, hq, hd, budget, p, s, smax, key_sketch=key_sketch,
+                       hook_order=_hip.ORDER_ANY)
+    ks, vs = rand_bf16(rng, b, seq, hkv, hd), rand_bf16(rng, b, seq, hkv, hd)
+    cache.prefill_update_kv_cache(dev_bf16(ks), dev_bf16(vs), 0)
+    p_len, s_len, lo, hi = orc.region_split(seq, p, s)
+    q = rand_bf16(rng, b, 1, hq * hd)
+    cache.decode_pre_query_operation(dev_bf16(q))
+    cache.decode_query_kvcache(0)
+    cache.decode_post_query_operation(0)
+    kc, vc = cache.get_kvcache(0)
+    kc, vc = np_u16(kc), np_u16(vc)
+    qmean = orc.group_mean_bf16(q.reshape(b, hq, hd), hkv)
+    ids = cache.idx[0].cpu().numpy()[:, :budget].astype(np.int64)
+    for h in range(hkv):
+        K, V = ks[0, :, h], vs[0, :, h]
+        sel = orc.topk_select(orc.scores_f32(qmean[0, h], K[lo:hi]), budget, orc.MODE_REF_DIST)
+        assert np.array_equal(np.sort(ids[h]), np.sort(sel))
+        assert np.array_equal(kc[0, :budget, h], K[ids[h] + lo]) and np.array_equal(vc[0, :budget, h], V[ids[h] + lo])
+        rest = orc.attended_rows(sel, p_len, hi, seq)[budget:]
+        assert np.array_equal(kc[0, budget:budget + p_len + s_len, h], K[rest])
+
+
 @pytest.mark.parametrize("key_mode", ["ref_dist", "ip"])
 def test_diffcache_decode_attention_matches_oracle_over_steps(key_mode):
     rng = np.random.default_rng(20)
