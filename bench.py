@@ -173,6 +173,7 @@ class DecodeWorkload:
         self.scores = None
         self.stream = torch.cuda.Stream(device=dev)     # default priority
         self.clean = False
+        self.calls = {}
 
     def layer(self, l: int, scan: str, mode: int, ev=None, route_only: bool = False):
         """One dc_decode_layer call.  scan: "sketch", "bf16" or "dense" (fp32 scores +
@@ -181,13 +182,16 @@ class DecodeWorkload:
         k, v, q, nk, nv = self.layers[l]
         if scan == "dense" and self.scores is None:
             self.scores = self.torch.empty((self.n_units, self.region), dtype=self.torch.float32, device=self.dev)
-        args = (q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
-                self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv)
-        kw = dict(mode=mode, order=hip.ORDER_ANY, select_state_ready=self.clean and scan != "dense",
-                  scan_events=ev, sketch=self.sketches[l] if scan == "sketch" else None)
+        call = self.calls.get((l, scan, mode))
+        if call is None:
+            # the argument struct of a layer is built once; a step only calls dc_decode_layer
+            call = self.calls[(l, scan, mode)] = hip.LayerCall(
+                q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
+                self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv,
+                mode=mode, order=hip.ORDER_ANY, sketch=self.sketches[l] if scan == "sketch" else None)
         if route_only:
-            return hip.decode_layer_route(*args, **kw)
-        hip.decode_layer(*args, **kw)
+            return call.route()
+        call(select_state_ready=self.clean and scan != "dense", scan_events=ev)
         self.clean = scan != "dense"
 
     def measure(self, scan: str, mode: int, steps: int, warmup: int, event_stride: int = 4,
@@ -205,29 +209,36 @@ class DecodeWorkload:
             return evs
 
         def step(evs):
-            with torch.cuda.stream(self.stream):
-                for l in range(L):
-                    ev = None
-                    if evs is not None and l in timed:
-                        j = timed.index(l)
-                        ev = (evs[2 * j], evs[2 * j + 1])
-                    self.layer(l, scan, mode, ev)
+            for l in range(L):
+                ev = None
+                if evs is not None and l in timed:
+                    j = timed.index(l)
+                    ev = (evs[2 * j], evs[2 * j + 1])
+                self.layer(l, scan, mode, ev)
 
-        events = [new_events(2 * len(timed)) for _ in range(steps)]
-        marks = new_events(steps + 1)
+        # A step of few layers is shorter than the events that time it cost (an event is a packet of
+        # its own in the queue): then only every `group`-th step carries the in-place event pairs
+        # and the per-step marks bracket `group` steps.
+        group = 1 if L >= 8 else 8
+        n_marks = steps // group if steps >= group else 1
+        group = group if steps >= group else steps
+        events = [new_events(2 * len(timed)) for _ in range(n_marks)]
+        marks = new_events(n_marks + 1)
         torch.cuda.synchronize()
-        for _ in range(warmup):
-            step(None)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        marks[0].record(self.stream)
-        for s in range(steps):
-            step(events[s])
-            marks[s + 1].record(self.stream)
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+        with torch.cuda.stream(self.stream):
+            for _ in range(warmup):
+                step(None)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            marks[0].record()
+            for s in range(steps):
+                step(events[s // group] if s % group == 0 and s // group < n_marks else None)
+                if (s + 1) % group == 0 and (s + 1) // group <= n_marks:
+                    marks[(s + 1) // group].record()
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - t0
         ms_per_step = elapsed * 1e3 / steps
-        per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(steps))
+        per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 / group for i in range(n_marks))
 
         def pct(p):
             return per_step_us[min(len(per_step_us) - 1, int(p * len(per_step_us)))]
@@ -247,8 +258,7 @@ class DecodeWorkload:
                 with torch.cuda.stream(self.stream):
                     flush.fill_(s_i & 0xff)
                     c0.record()
-                step(None)
-                with torch.cuda.stream(self.stream):
+                    step(None)
                     c1.record()
                 torch.cuda.synchronize()
                 samples.append(c0.elapsed_time(c1) * 1e3)

@@ -575,6 +575,29 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
     return out
 
 
+class LayerCall:
+    """A decode_layer call with its argument struct built once: a serving loop that calls the same
+    layer with the same tensors every step pays the checks of decode_layer once and a bare
+    dc_decode_layer call afterwards.  The tensors are kept alive by the object."""
+
+    def __init__(self, *args, **kwargs) -> None:
+        self.args = _layer_args(*args, **kwargs)
+
+    def __call__(self, select_state_ready: Optional[bool] = None,
+                 scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None) -> None:
+        a = self.args
+        if select_state_ready is not None:
+            a.select_state_ready = 1 if select_state_ready else 0
+        if scan_events is not None:
+            a.ev_scan_begin, a.ev_scan_end = scan_events[0].cuda_event, scan_events[1].cuda_event
+        else:
+            a.ev_scan_begin, a.ev_scan_end = None, None
+        _check(lib.dc_decode_layer(C.byref(a), _stream()))
+
+    def route(self) -> int:
+        return int(lib.dc_decode_layer_route(C.byref(self.args)))
+
+
 ROUTE_ATTEND_ONLY, ROUTE_DENSE, ROUTE_STREAM, ROUTE_SKETCH, ROUTE_ONE_KERNEL = range(5)
 
 

@@ -167,3 +167,25 @@ def test_small_context_bounded_wait_is_reported():
     finally:
         hip.lib.dc_set_wait_limit(0)
     run_case(k, v, q, None, None, n_ctx, 512, 4, 64, orc.MODE_REF_DIST, reps=2, ws=ws)
+
+
+def test_prepared_layer_call_equals_decode_layer():
+    """hip.LayerCall builds the argument struct once; calling it equals decode_layer."""
+    rng = np.random.default_rng(305)
+    b, hq, hkv, hd, n_ctx, budget = 1, 8, 2, 128, 20000, 256
+    k, v, q = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hq, hd)
+    kd, vd, qd = to_dev_bf16(k), to_dev_bf16(v), to_dev_bf16(q)
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+    ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, budget, hq // hkv, hd, budget + 69), DEV)
+    for order in (hip.ORDER_ANY, hip.ORDER_BEST):
+        idx = [torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV) for _ in range(2)]
+        out = [torch.empty((b, hq, hd), dtype=torch.bfloat16, device=DEV) for _ in range(2)]
+        hip.decode_layer(qd, kd, vd, p_len, hi, s_len, budget, None, idx[0], out[0], ws, order=order)
+        call = hip.LayerCall(qd, kd, vd, p_len, hi, s_len, budget, None, idx[1], out[1], ws, order=order)
+        assert call.route() == (hip.ROUTE_ONE_KERNEL if order == hip.ORDER_ANY else hip.ROUTE_STREAM)
+        call(select_state_ready=True)
+        call(select_state_ready=True)
+        torch.cuda.synchronize()
+        assert torch.equal(torch.sort(idx[0], dim=1).values, torch.sort(idx[1], dim=1).values)
+        # (the one-kernel route deals rows to blocks in arrival order: equal within float rounding)
+        assert torch.allclose(out[0].float(), out[1].float(), atol=2e-3, rtol=2.0 ** -7)
