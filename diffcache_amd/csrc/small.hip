@@ -11,8 +11,10 @@
 //      histogram of ordering-key buckets to the unit's          -- barrier (arrival counter) --
 //   2  every block derives the threshold bucket from the complete histogram, emits the ids of
 //      its rows in better buckets and writes its rows of the threshold bucket into slots of
-//      the unit's candidate list.  The histogram says how many candidates there are, and an
-//      unwritten slot reads "empty", so the list itself tells a reader when it is complete
+//      the unit's candidate list.  No slot is reserved through a counter: what the block's
+//      addition to a bucket of the histogram returned is its place among the unit's rows of
+//      that bucket.  The histogram also says how many candidates there are, and an unwritten
+//      slot reads "empty", so the list itself tells a reader when it is complete
 //   3  every block ranks its own candidates among all of the unit's: those among the
 //      k - (rows in better buckets) smallest (key, id) pairs are in (ties to the lower id: the
 //      kept set of search_bruteforce, nsw.rs:592-630).  (Candidates by the thousand -- equal
@@ -164,10 +166,12 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     constexpr int R = rows_per_group(G);
     __shared__ __align__(16) unsigned char smem[small_lds_bytes<HD, G>()];
     __shared__ uint32_t lhist[DC_HIST_BINS];
+    __shared__ uint32_t lbase[DC_HIST_BINS];  // what this block's additions to the unit's histogram returned
+    __shared__ uint32_t lpre[DC_HIST_BINS];   // exclusive prefix of the unit's histogram
     __shared__ uint32_t wtot[kThreads / 64 + 1];
     __shared__ uint32_t sres[3];
-    __shared__ uint32_t s_cnt[4];   // own winners, own candidates, write cursors
-    __shared__ uint32_t s_base[2];  // global slots reserved for this block's ids / candidates
+    __shared__ uint32_t s_cnt[4];   // [2]: this block's selected rows so far
+    __shared__ uint32_t s_base[2];  // scratch of the radix select
     __shared__ uint32_t s_flag;
     float *s_scores = reinterpret_cast<float *>(smem);
     unsigned long long *s_cand = reinterpret_cast<unsigned long long *>(smem);
@@ -223,9 +227,12 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
         }
     }
     __syncthreads();
+    // What an addition returns -- the rows of that bucket counted before this block's -- is the
+    // block's place among the unit's rows of the bucket: every selected id and every candidate
+    // gets its slot from the histogram, and no other counter is needed.
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
         const uint32_t c = lhist[i];
-        if (c) atomicAdd(&hu[i], c);
+        lbase[i] = c ? atomicAdd(&hu[i], c) : 0u;
     }
 
     // ---------------- 2: threshold bucket; ids of better buckets, candidates of the threshold bucket ----------------
@@ -247,56 +254,41 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
         }
         __syncthreads();
         const uint32_t kk = (uint32_t)a.k_eff;
-        if (excl < kk && kk <= excl + sum) {
-            uint32_t run = excl;
-            bool done = false;
+        uint32_t run = excl;
+        bool done = !(excl < kk && kk <= excl + sum);
 #pragma unroll
-            for (int i = 0; i < kBinsPerThread; ++i) {
-                if (!done && run + bins[i] >= kk) {
-                    sres[0] = tid * kBinsPerThread + i;
-                    sres[1] = run;
-                    sres[2] = bins[i];
-                    done = true;
-                }
-                run += bins[i];
+        for (int i = 0; i < kBinsPerThread; ++i) {
+            lpre[tid * kBinsPerThread + i] = run;  // rows of the unit in better buckets
+            if (!done && run + bins[i] >= kk) {
+                sres[0] = tid * kBinsPerThread + i;
+                sres[1] = run;
+                sres[2] = bins[i];
+                done = true;
             }
+            run += bins[i];
         }
         __syncthreads();
         tb = sres[0];
         c_less = sres[1];
         n_cand = sres[2];  // rows of the threshold bucket in the whole unit
     }
-    // count, reserve the global slots, then write
-    {
-        uint32_t nw = 0, nc = 0;
-        for (int i = tid; i < n_own; i += kThreads) {
-            uint32_t key, bucket;
-            dc_key_bucket(s_scores[i], a.mode, key, bucket);
-            nw += bucket < tb ? 1u : 0u;
-            nc += bucket == tb ? 1u : 0u;
-        }
-        if (nw) atomicAdd(&s_cnt[0], nw);
-        if (nc) atomicAdd(&s_cnt[1], nc);
-    }
+    const uint32_t n_oc = tb < (uint32_t)DC_HIST_BINS ? lhist[tb] : 0u;    // this block's rows of that bucket
+    const uint32_t base_c = tb < (uint32_t)DC_HIST_BINS ? lbase[tb] : 0u;  // and their first slot in the list
     __syncthreads();
-    const uint32_t n_win1 = s_cnt[0], n_oc = s_cnt[1];
-    if (tid == 0) s_base[0] = n_win1 ? atomicAdd(&st->win_cnt, n_win1) : 0u;  // (two waves: the two
-    if (tid == 64) s_base[1] = n_oc ? atomicAdd(&st->cand_cnt, n_oc) : 0u;    //  round trips overlap)
+    for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;  // from here on: rows of a bucket placed so far
     __syncthreads();
     uint32_t *io = a.idx_out + (int64_t)unit * a.idx_stride;
     unsigned long long *cl = a.cand + (int64_t)unit * a.n_rows;
-    const uint32_t base_c = s_base[1];
     for (int i = tid; i < n_own; i += kThreads) {
         uint32_t key, bucket;
         dc_key_bucket(s_scores[i], a.mode, key, bucket);
         const uint32_t id = (uint32_t)(r0 + i);
         if (bucket < tb) {
-            const uint32_t p = atomicAdd(&s_cnt[2], 1u);
-            own_win[p] = id;
-            const uint32_t slot = s_base[0] + p;
+            own_win[atomicAdd(&s_cnt[2], 1u)] = id;
+            const uint32_t slot = lpre[bucket] + lbase[bucket] + atomicAdd(&lhist[bucket], 1u);
             if (slot < (uint32_t)a.k_eff) io[slot] = id;
         } else if (bucket == tb) {
-            const uint32_t slot = base_c + atomicAdd(&s_cnt[3], 1u);
+            const uint32_t slot = base_c + atomicAdd(&lhist[bucket], 1u);
             if (slot < n_cand) st_agent_u64(cl + slot, ((unsigned long long)key << 32) | id);
         }
     }
@@ -349,11 +341,10 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
                 rank += (t.x < mine ? 1u : 0u) + (t.y < mine ? 1u : 0u);
             }
             for (uint32_t off = 1; off < T; off <<= 1) rank += __shfl_xor(rank, (int)off, 64);
-            if (active && sub == 0 && rank < need) {
+            if (active && sub == 0 && rank < need) {  // ranks are distinct: the rank is the slot
                 const uint32_t id = (uint32_t)mine;
                 own_win[atomicAdd(&s_cnt[2], 1u)] = id;
-                const uint32_t gs = atomicAdd(&st->win_cnt, 1u);
-                if (gs < (uint32_t)a.k_eff) io[gs] = id;
+                io[c_less + rank] = id;
             }
         }
     } else {
@@ -442,7 +433,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
             const uint32_t key = (uint32_t)(c >> 32), id = (uint32_t)c;
             if (key < cut_key || (key == cut_key && id <= cut_id)) {
                 own_win[atomicAdd(&s_cnt[2], 1u)] = id;
-                const uint32_t gs = atomicAdd(&st->win_cnt, 1u);
+                const uint32_t gs = c_less + atomicAdd(&st->win_cnt, 1u);
                 if (gs < (uint32_t)a.k_eff) io[gs] = id;
             }
         }
@@ -586,7 +577,6 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) dc_st_agent(hu + i, 0u);
     for (uint32_t i = tid; i < n_cand; i += kThreads) st_agent_u64(cl + i, kEmpty);
     if (tid == 0) {
-        dc_st_agent(&st->cand_cnt, 0u);
         dc_st_agent(&st->win_cnt, 0u);
         dc_st_agent(&st->sync_cnt, 0u);
     }
