@@ -8,6 +8,7 @@ constexpr int kFinalThreads = 1024;
 constexpr int kRadixBits = 11;
 constexpr int kRadixBins = 1 << kRadixBits;
 constexpr int kScanBatch = 8;  // items of a list that a thread fetches before it looks at any
+constexpr int kScanShort = 8192;  // lists up to this length sit in LDS (kCandLds of the callers): plain loops
 
 // inclusive scan over the lanes of a wave
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
@@ -44,6 +45,10 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, 
 // f(key, id) for every entry of a (key, id) list, kScanBatch entries of a thread in flight.
 template <int NT, typename F>
 __device__ __forceinline__ void dc_for_each_pair(const uint32_t *ck, const uint32_t *ci, uint32_t n, F f) {
+    if (n <= (uint32_t)kScanShort) {
+        for (uint32_t i = threadIdx.x; i < n; i += NT) f(ck[i], ci[i]);
+        return;
+    }
     for (uint32_t i0 = threadIdx.x; i0 < n; i0 += kScanBatch * NT) {
         uint32_t key[kScanBatch], id[kScanBatch];
 #pragma unroll
@@ -75,10 +80,17 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
     for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
     __syncthreads();
     const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
+    if (n <= (uint32_t)kScanShort) {  // a list that the caller keeps in LDS: nothing to hide
+        for (uint32_t i = tid; i < n; i += kFinalThreads) {
+            uint32_t v;
+            if (get(i, &v) && ((v & himask) == (prefix & himask)))
+                atomicAdd(&lh[(v >> shift) & ((1u << width) - 1u)], 1u);
+        }
+    }
     // kScanBatch items of a thread are fetched before any is looked at: with one load per
     // iteration a long list costs a memory round trip per item and thread.  A wave whose lanes
     // all hit one bin (long runs of equal keys) adds its count once.
-    for (uint32_t i0 = tid; i0 < n; i0 += kScanBatch * kFinalThreads) {
+    for (uint32_t i0 = tid; n > (uint32_t)kScanShort && i0 < n; i0 += kScanBatch * kFinalThreads) {
         uint32_t v[kScanBatch];
         bool in[kScanBatch];
 #pragma unroll
@@ -166,7 +178,9 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
     __syncthreads();
     const uint32_t k0 = ck[0];
     uint32_t diff = 0;
-    for (uint32_t i0 = tid; i0 < n_c; i0 += kScanBatch * kFinalThreads) {
+    if (n_c <= (uint32_t)kScanShort)
+        for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
+    for (uint32_t i0 = tid; n_c > (uint32_t)kScanShort && i0 < n_c; i0 += kScanBatch * kFinalThreads) {
         uint32_t v[kScanBatch];
 #pragma unroll
         for (int u = 0; u < kScanBatch; ++u) {
