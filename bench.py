@@ -39,8 +39,10 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes one scan launch of configuration 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # scaled by a known-size copy kernel: counts x 2 KiB read + counts x 1 KiB written.  Taken
 # once, when the profile summaries kept with this repository were made -- not in this run.
-SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_722 * 2048 + 13_249 * 1024,
-                            "bf16": 1_053_933 * 2048 + 12_570 * 1024}
+SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_752 * 2048 + 13_214 * 1024,
+                            "bf16": 1_048_550 * 2048 + 11_289 * 1024}
+# the one-kernel route of configuration 2 (small_layer_kernel), same counters
+LAYER_TRAFFIC_PROFILED_C2 = 35_234 * 2048 + 1_477 * 1024
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
@@ -314,8 +316,9 @@ class DecodeWorkload:
             "achieved_8d": rows_bytes_8d / (scan_ms * 1e-3) / 1e9,
             "frac_8d": rows_bytes_8d / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         }
-        if self.name == "c3" and scan in SCAN_TRAFFIC_PROFILED_C3:
-            roofline["traffic"] = SCAN_TRAFFIC_PROFILED_C3[scan]
+        one_kernel = kernel.startswith("small_layer_kernel")
+        if (self.name == "c3" and scan in SCAN_TRAFFIC_PROFILED_C3) or (self.name == "c2" and one_kernel):
+            roofline["traffic"] = LAYER_TRAFFIC_PROFILED_C2 if one_kernel else SCAN_TRAFFIC_PROFILED_C3[scan]
             roofline["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE when the committed profile " \
                                          "summaries were taken, not measured in this run"
         s_per_step = ms_per_step * 1e-3
