@@ -8,7 +8,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kRowsPerBlockStep = 256;
 constexpr int kBigSteps = 8;       // 2048 rows per large block
-constexpr int kSmallChunks = 32;   // leading 256-row blocks per unit
+constexpr int kSmallChunks = 16;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
 constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
 constexpr int kSharedPollUnits = 8;   // sketch scan: up to this many units, one wave per block polls
