@@ -354,6 +354,9 @@ int dc_decode_layer(const dc_layer_args *args, void *stream);
  * that kernel).  Its waits between blocks are bounded; dc_decode_layer_status waits for
  * `stream` and returns DC_EDEVICE if a wait of the last calls on this workspace ran out (never
  * observed; the outputs would be invalid), DC_OK otherwise.  `args` as in the call it checks.
+ * The kernel counts on all its blocks running at the same time (two per CU): it may share the
+ * GPU with short kernels of other streams, which only delay it, but not with kernels that keep
+ * CUs occupied for good -- then its waits run out (after about a second each) instead of ending.
  * No counterpart in the reference, whose layers run on the CPU pool (lib.rs:352-369).
  */
 int dc_decode_layer_status(const dc_layer_args *args, void *stream);
