@@ -189,3 +189,56 @@ def test_prepared_layer_call_equals_decode_layer():
         assert torch.equal(torch.sort(idx[0], dim=1).values, torch.sort(idx[1], dim=1).values)
         # (the one-kernel route deals rows to blocks in arrival order: equal within float rounding)
         assert torch.allclose(out[0].float(), out[1].float(), atol=2e-3, rtol=2.0 ** -7)
+
+
+def test_small_context_agrees_with_the_kernel_chain_on_random_cases():
+    """120 random shapes, budgets, key modes and data laws: the one-kernel route (ids in any
+    order) against the chain of kernels that the same call takes when the ids are asked best
+    first.  Same id sets, outputs within bf16 rounding of each other."""
+    rng = np.random.default_rng(306)
+    n_one = 0
+    for case in range(120):
+        hd = int(rng.choice([64, 128, 256]))
+        g = int(rng.choice([1, 2, 4, 7, 8]))
+        hkv = int(rng.integers(1, 7))
+        b = int(rng.integers(1, 4))
+        p, s = int(rng.integers(0, 6)), int(rng.integers(0, 40))
+        region = int(rng.choice([1, 2, 17, 255, 256, 257, 1000, 3000, 7000, 12000]))
+        budget = int(rng.choice([1, 8, 100, 512, 2048, region, region + 5]))
+        mode = int(rng.integers(0, 2))
+        law = rng.choice(["normal", "integers", "constant", "two_values"])
+        n_ctx = p + region + s
+        shape = (b, hkv, n_ctx, hd)
+        if law == "normal":
+            kf = rng.standard_normal(shape)
+        elif law == "integers":
+            kf = rng.integers(-2, 3, shape)
+        elif law == "constant":
+            kf = np.broadcast_to(rng.standard_normal((b, hkv, 1, hd)), shape)
+        else:
+            kf = np.where(rng.random((b, hkv, n_ctx, 1)) < 0.5, 1.0, -1.0) * rng.standard_normal((b, hkv, 1, hd))
+        k = to_dev_bf16(orc.f32_to_bf16(np.ascontiguousarray(kf, dtype=np.float32)))
+        v = to_dev_bf16(rand_bf16(rng, *shape))
+        q = to_dev_bf16(rand_bf16(rng, b, hkv * g, hd))
+        nk, nv = to_dev_bf16(rand_bf16(rng, b, hkv, hd)), to_dev_bf16(rand_bf16(rng, b, hkv, hd))
+        k_eff = min(budget, region)
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, region, budget, g, hd, k_eff + p + s + 1), DEV)
+        res = {}
+        for order in (hip.ORDER_ANY, hip.ORDER_BEST):
+            idx = torch.full((b * hkv, max(budget, 1)), -1, dtype=torch.int32, device=DEV)
+            out = torch.empty((b, hkv * g, hd), dtype=torch.bfloat16, device=DEV)
+            lse = torch.empty((b, hkv * g), dtype=torch.float32, device=DEV)
+            args = (q, k, v, p, p + region, s, budget, None, idx, out, ws, nk, nv)
+            kw = dict(lse=lse, mode=mode, order=order)
+            route = hip.decode_layer_route(*args, **kw)
+            hip.decode_layer(*args, **kw)
+            hip.decode_layer_status(*args, **kw)
+            res[order] = (torch.sort(idx[:, :k_eff], dim=1).values.cpu(), out.float().cpu(), lse.cpu(), route)
+        one, chain = res[hip.ORDER_ANY], res[hip.ORDER_BEST]
+        n_one += one[3] == hip.ROUTE_ONE_KERNEL
+        tag = (case, hd, g, hkv, b, p, s, region, budget, mode, str(law))
+        assert chain[3] != hip.ROUTE_ONE_KERNEL, tag
+        assert torch.equal(one[0], chain[0]), tag
+        assert torch.allclose(one[1], chain[1], atol=4e-3, rtol=2.0 ** -6), tag
+        assert torch.allclose(one[2], chain[2], atol=1e-3, rtol=1e-4), tag
+    assert n_one >= 100       # (a group size whose kernel does not fit twice on a CU takes the chain)
