@@ -31,6 +31,7 @@
 #include "dc_attn.h"
 #include "dc_fused.h"
 #include <atomic>
+#include <cstdlib>
 #include <mutex>
 
 namespace {
@@ -759,6 +760,13 @@ extern "C" void dc_set_wait_limit(int polls) { g_small_wait_limit.store(polls > 
 // once (the blocks of a unit wait for each other), a block's rows must fit its LDS, and the
 // merge must hold the (m, l) pairs of a unit's blocks.
 bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd) {
+    // DIFFCACHE_ONE_KERNEL=0 in the environment (read once) switches the route off, for processes
+    // that share the GPU with kernels that never leave their CUs
+    static const bool enabled = [] {
+        const char *e = std::getenv("DIFFCACHE_ONE_KERNEL");
+        return !(e && e[0] == '0' && e[1] == 0);
+    }();
+    if (!enabled) return false;
     if (k_eff < 1 || group < 1 || group > 8 || !(hd == 64 || hd == 128 || hd == 256)) return false;
     const SmallPlan p = plan_small(n_units, region);
     if (!p.ok || p.bpu * group * 2 > kSmallMl) return false;

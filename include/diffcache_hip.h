@@ -357,6 +357,7 @@ int dc_decode_layer(const dc_layer_args *args, void *stream);
  * The kernel counts on all its blocks running at the same time (two per CU): it may share the
  * GPU with short kernels of other streams, which only delay it, but not with kernels that keep
  * CUs occupied for good -- then its waits run out (after about a second each) instead of ending.
+ * DIFFCACHE_ONE_KERNEL=0 in the environment of the process switches the route off.
  * No counterpart in the reference, whose layers run on the CPU pool (lib.rs:352-369).
  */
 int dc_decode_layer_status(const dc_layer_args *args, void *stream);
