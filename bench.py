@@ -39,8 +39,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes one scan launch of configuration 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # scaled by a known-size copy kernel: counts x 2 KiB read + counts x 1 KiB written.  Taken
 # once, when the profile summaries kept with this repository were made -- not in this run.
-SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_752 * 2048 + 13_214 * 1024,
-                            "bf16": 1_048_550 * 2048 + 11_289 * 1024}
+SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_698 * 2048 + 16_457 * 1024,
+                            "bf16": 1_048_497 * 2048 + 14_402 * 1024}
 # the one-kernel route of configuration 2 (small_layer_kernel), same counters
 LAYER_TRAFFIC_PROFILED_C2 = 35_234 * 2048 + 1_477 * 1024
 

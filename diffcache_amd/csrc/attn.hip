@@ -28,7 +28,7 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(AttnArgs a) {
     sh.red = s_mem;
     sh.l = s_mem + kAttnWaves * G;
     sh.acc = s_mem + 2 * kAttnWaves * G;
-    dc_attn_split<HD, G, false>(a, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, sh);
+    dc_attn_split<HD, G>(a, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, sh);
 }
 
 // out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block

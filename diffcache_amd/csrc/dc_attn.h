@@ -92,9 +92,8 @@ struct AttnShared {
 template <int HD, int G>
 constexpr int attn_shared_floats() { return kAttnWaves * G * 2 + kAttnWaves * G * HD; }
 
-// One split of one unit.  COHERENT: the ids were written, and the partials will be read, by
-// other blocks of the same kernel (see dc_ld_agent).
-template <int HD, int G, bool COHERENT>
+// One split of one unit.
+template <int HD, int G>
 __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int split, const AttnShared &sh) {
     constexpr int LPR = HD / 8;
     constexpr int NG = kAttnThreads / LPR;  // row groups per block
@@ -139,7 +138,7 @@ __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int s
         if (ok[t]) {
             if (vj < n_idx) {
                 const uint32_t *ip = a.idx + (int64_t)unit * a.idx_stride + vj;
-                r = (uint32_t)(a.region_lo + (COHERENT ? dc_ld_agent(ip) : *ip));
+                r = (uint32_t)(a.region_lo + *ip);
             } else if (vj < n_idx + n_sink) {
                 r = (uint32_t)(vj - n_idx);
             } else if (vj < n_idx + n_sink + n_recent) {
@@ -258,8 +257,7 @@ __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int s
         float s = s_acc[0][o];
 #pragma unroll
         for (int w2 = 1; w2 < kAttnWaves; ++w2) s += s_acc[w2][o];
-        if (COHERENT) dc_st_agent(a.ws_acc + slot * (G * HD) + o, s);
-        else a.ws_acc[slot * (G * HD) + o] = s;
+        a.ws_acc[slot * (G * HD) + o] = s;
     }
     if (tid < G) {
         float l = s_l[0][tid];
@@ -269,13 +267,8 @@ __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int s
 #pragma unroll
         for (int w2 = 1; w2 < kAttnWaves; ++w2) mm = fmaxf(mm, s_red[w2][tid]);
         float *ml = a.ws_ml + (slot * G + tid) * 2;
-        if (COHERENT) {
-            dc_st_agent(ml + 0, mm);
-            dc_st_agent(ml + 1, l);
-        } else {
-            ml[0] = mm;
-            ml[1] = l;
-        }
+        ml[0] = mm;
+        ml[1] = l;
     }
 }
 
