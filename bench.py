@@ -190,7 +190,10 @@ class DecodeWorkload:
             call = self.calls[(l, scan, mode)] = hip.LayerCall(
                 q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
                 self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv,
-                mode=mode, order=hip.ORDER_ANY, sketch=self.sketches[l] if scan == "sketch" else None)
+                mode=mode, order=hip.ORDER_ANY, sketch=self.sketches[l] if scan == "sketch" else None,
+                # this process has the GPU to itself and one stream: short contexts may run as one
+                # kernel inside the captured step as well
+                one_kernel=hip.ONE_KERNEL_EXCLUSIVE)
         if route_only:
             return call.route()
         call(select_state_ready=self.clean and scan != "dense", scan_events=ev)

@@ -15,6 +15,7 @@ import torch
 
 MODE_IP = 0
 MODE_REF_DIST = 1
+ONE_KERNEL_AUTO, ONE_KERNEL_EXCLUSIVE, ONE_KERNEL_NEVER = 0, 1, -1
 ORDER_ANY = 0
 ORDER_BEST = 1
 ORDER_INDEX = 2
@@ -29,7 +30,8 @@ SYMBOLS = (
     "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
     "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_gather_attn_static_bf16", "dc_append_kv_bf16",
     "dc_step_advance", "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
-    "dc_decode_layer_status", "dc_set_wait_limit", "dc_decode_layer_route",
+    "dc_decode_layer_status", "dc_set_wait_limit", "dc_decode_layer_route", "dc_last_route",
+    "dc_decode_layer_errors", "dc_one_kernel_guard",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
     "dc_score_select_workspace_bytes", "dc_select_state_init", "dc_score_prune_bf16",
     "dc_sparse_select", "dc_score_select_bf16",
@@ -60,6 +62,7 @@ class LayerArgs(C.Structure):
         ("sketch_batch_stride", C.c_int64), ("sketch_head_stride", C.c_int64),
         ("sketch_row_stride", C.c_int64),
         ("n_recent_dev", C.c_void_p),
+        ("one_kernel", C.c_int),
     ]
 
 
@@ -91,6 +94,9 @@ def _load() -> C.CDLL:
         "dc_decode_layer_status": (i, [C.POINTER(LayerArgs), p]),
         "dc_set_wait_limit": (None, [i]),
         "dc_decode_layer_route": (i, [C.POINTER(LayerArgs)]),
+        "dc_last_route": (i, []),
+        "dc_decode_layer_errors": (C.c_uint, []),
+        "dc_one_kernel_guard": (i, [i, i, i, i, i]),
         "dc_pq_build_lut": (i, [p, p, p, i, i, i, i, p]),
         "dc_pq_adc_scan": (i, [p, p, p, p, i, i, i, i64, p]),
         "dc_score_gathered_bf16": (i, [p, p, p, p, i, i, i, i64, i, i64, i64, i64, i64, i64, p]),
@@ -508,7 +514,8 @@ def layer_workspace_bytes(n_units: int, n_region: int, budget: int, group: int, 
 
 def _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
                 new_k=None, new_v=None, lse=None, mode=MODE_REF_DIST, order=ORDER_ANY, scale=None,
-                select_state_ready=False, scan_events=None, sketch=None, n_recent_dev=None) -> "LayerArgs":
+                select_state_ready=False, scan_events=None, sketch=None, n_recent_dev=None,
+                one_kernel=ONE_KERNEL_AUTO) -> "LayerArgs":
     """struct dc_layer_args from tensors (the arguments of decode_layer), with their checks."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
@@ -551,6 +558,7 @@ def _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores
         a.sketch_resid = _dev(sketch.resid, "resid")
         a.sketch_batch_stride, a.sketch_head_stride, a.sketch_row_stride = c.stride(0), c.stride(1), c.stride(2)
     a.n_recent_dev = _counter(n_recent_dev)
+    a.one_kernel = one_kernel
     a._keep = (q, store_k, store_v, new_k, new_v, out, lse, scores, idx_out, workspace, sketch, n_recent_dev)
     return a
 
@@ -564,13 +572,16 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
                  select_state_ready: bool = False,
                  scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
                  sketch: Optional["Sketch"] = None,
-                 n_recent_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 n_recent_dev: Optional[torch.Tensor] = None,
+                 one_kernel: int = ONE_KERNEL_AUTO) -> torch.Tensor:
     """score -> select -> attend for one layer, enqueued on the current stream.
     ``n_recent_dev``: the suffix length as a device-side int32 (``n_recent`` = capacity).
     ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
-    ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result)."""
+    ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result).
+    ``one_kernel``: ONE_KERNEL_* policy for short contexts (see the header)."""
     a = _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
-                    new_k, new_v, lse, mode, order, scale, select_state_ready, scan_events, sketch, n_recent_dev)
+                    new_k, new_v, lse, mode, order, scale, select_state_ready, scan_events, sketch, n_recent_dev,
+                    one_kernel)
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
 
@@ -599,6 +610,16 @@ class LayerCall:
 
 
 ROUTE_ATTEND_ONLY, ROUTE_DENSE, ROUTE_STREAM, ROUTE_SKETCH, ROUTE_ONE_KERNEL = range(5)
+
+
+def last_route() -> int:
+    """The route the last decode_layer call of this thread actually took (a ROUTE_* value)."""
+    return int(lib.dc_last_route())
+
+
+def decode_layer_errors() -> int:
+    """Failures of the one-kernel route seen so far in this process (no synchronisation)."""
+    return int(lib.dc_decode_layer_errors())
 
 
 def decode_layer_route(*args, **kwargs) -> int:

@@ -6,6 +6,7 @@
 #include <string.h>
 
 static thread_local char g_err[512] = "";
+static thread_local int g_last_route = DC_ROUTE_ATTEND_ONLY;
 
 void dc_set_error(const char *fmt, ...) {
     va_list ap;
@@ -17,6 +18,8 @@ void dc_set_error(const char *fmt, ...) {
 extern "C" int dc_version(void) { return DC_VERSION; }
 
 extern "C" const char *dc_last_error(void) { return g_err; }
+
+extern "C" int dc_last_route(void) { return g_last_route; }
 
 namespace {
 
@@ -31,6 +34,7 @@ struct LayerWs {
     size_t topk_bytes;
     void *attn;
     size_t attn_bytes;
+    void *small_cand;  // candidate lists of the one-kernel route (shapes it can take only)
     size_t bytes;
 };
 
@@ -55,6 +59,8 @@ LayerWs carve_layer(void *base, int n_units, int n_region, int budget, int group
         w.attn_bytes = dc_align_up(a > b ? a : b, 256);
     }
     off += w.attn_bytes;
+    w.small_cand = p + off;
+    off += dc_small_cand_bytes(n_units, n_region);
     w.bytes = off;
     return w;
 }
@@ -93,20 +99,37 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     int rc;
     const uint16_t *k_region = (const uint16_t *)a->k + (int64_t)a->n_sink * a->kv_row_stride;
+    // The caller's word that the select state is ready counts unless a kernel of the one-kernel
+    // route has reported a failure since this workspace was last initialised.
+    int ready = a->select_state_ready;
+    if (k_eff > 0 && !a->scores) {
+        if (ready && !dc_ws_state_trusted(a->workspace)) ready = 0;
+        if (!ready) dc_ws_state_initialised(a->workspace);
+    }
+    g_last_route = k_eff <= 0 ? DC_ROUTE_ATTEND_ONLY
+                              : (a->scores ? DC_ROUTE_DENSE : (a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM));
     if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY &&
         dc_small_supported(n_units, region, k_eff, a->group, a->hd)) {
         // short context: the whole layer in one kernel whose blocks are all resident (ids in no
-        // particular order); reads the bf16 keys, with or without a sketch
-        if (!a->select_state_ready) {
+        // particular order); reads the bf16 keys, with or without a sketch.  The state is set up
+        // for this route even when the call is sent down the chain below (another launch of the
+        // kernel is in flight on another stream, or the stream is being captured): the next call
+        // with these sizes may take the kernel and be told that the state is ready.
+        if (!ready) {
             rc = dc_select_state_init(n_units, region, a->budget, w.topk, w.topk_bytes, stream);
             if (rc) return rc;
-            rc = dc_small_state_init(n_units, region, a->budget, w.topk, stream);
+            rc = dc_small_state_init(n_units, region, w.small_cand, stream);
             if (rc) return rc;
+            ready = 1;
         }
         if (a->ev_scan_begin) (void)hipEventRecord((hipEvent_t)a->ev_scan_begin, st);
-        rc = dc_small_launch(a, region, k_eff, w.topk, w.attn, w.attn_bytes, stream);
-        if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
-        return rc;
+        rc = dc_small_try(a, region, k_eff, w.topk, w.small_cand, w.attn, w.attn_bytes, stream);
+        if (rc < 0) return rc;
+        if (rc == 1) {
+            if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
+            g_last_route = DC_ROUTE_ONE_KERNEL;
+            return DC_OK;
+        }
     }
     if (k_eff > 0 && !a->scores && a->sketch_codes) {
         // streaming select over the 8-bit sketch, exact rescoring of the kept rows
@@ -116,11 +139,11 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
             a->sketch_resid, a->q, a->idx_out, a->idx_unit_stride, a->n_b, a->n_h, region, a->hd,
             a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride, a->sketch_batch_stride,
             a->sketch_head_stride, a->sketch_row_stride, a->group, a->budget, a->mode, a->order,
-            a->select_state_ready, w.topk, w.topk_bytes, a->ev_scan_begin, a->ev_scan_end, stream);
+            ready, w.topk, w.topk_bytes, a->ev_scan_begin, a->ev_scan_end, stream);
         if (rc) return rc;
     } else if (k_eff > 0 && !a->scores) {
         // no dense scores wanted: streaming score + select
-        if (!a->select_state_ready) {
+        if (!ready) {
             rc = dc_select_state_init(n_units, region, a->budget, w.topk, w.topk_bytes, stream);
             if (rc) return rc;
         }
@@ -165,7 +188,9 @@ extern "C" int dc_decode_layer_route(const dc_layer_args *a) {
     const int k_eff = a->budget < region ? a->budget : region;
     if (n_units == 0 || k_eff <= 0) return DC_ROUTE_ATTEND_ONLY;
     if (a->scores) return DC_ROUTE_DENSE;
-    if (a->order == DC_ORDER_ANY && dc_small_supported(n_units, region, k_eff, a->group, a->hd)) return DC_ROUTE_ONE_KERNEL;
+    if (a->order == DC_ORDER_ANY && a->one_kernel != DC_ONE_KERNEL_NEVER &&
+        dc_small_supported(n_units, region, k_eff, a->group, a->hd))
+        return DC_ROUTE_ONE_KERNEL;
     return a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;
 }
 

@@ -43,9 +43,12 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
 // small.hip: a whole decode layer in one kernel, for short contexts
 bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd);
 size_t dc_small_workspace_bytes(int n_units, int region, int group, int hd);
-int dc_small_state_init(int n_units, int region, int budget, void *sel_ws, void *stream);
-int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws, void *attn_ws,
-                    size_t attn_ws_bytes, void *stream);
+size_t dc_small_cand_bytes(int n_units, int region);
+int dc_small_state_init(int n_units, int region, void *cand, void *stream);
+int dc_small_try(const dc_layer_args *a, int region, int k_eff, void *sel_ws, void *cand, void *attn_ws,
+                 size_t attn_ws_bytes, void *stream);
+bool dc_ws_state_trusted(const void *workspace);
+void dc_ws_state_initialised(const void *workspace);
 
 static inline bool dc_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline size_t dc_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

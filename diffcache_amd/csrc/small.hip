@@ -25,14 +25,20 @@
 //      shared state (histogram, counters, candidate slots) back to its initial values.
 //
 // A block that waits, waits for blocks that are resident too, so the wait ends; it is bounded
-// all the same.  Data that crosses blocks goes through agent-scope loads, stores and atomics:
-// the L2 caches of the eight XCDs are not coherent inside a kernel.  One such hand-over costs
+// all the same, and a wait that runs out cannot go unnoticed: the block sets the unit's error word
+// (which stays set until the host initialises the state again), tells the host through a word of
+// pinned host memory, and writes NaN over the unit's output rows and 0xffffffff over its ids; every
+// block of a later launch that finds the error word set does the same.  The host side keeps two
+// such launches from overlapping (they would starve each other of CUs): see dc_small_try.
+// Data that crosses blocks goes through agent-scope loads, stores and atomics: the L2 caches
+// of the eight XCDs are not coherent inside a kernel.  One such hand-over costs
 // about 1.5 to 2 us, and a layer is a chain of about ten of them after the 10 us of scoring.
 #include "dc_attn.h"
 #include "dc_fused.h"
 #include <atomic>
 #include <cstdlib>
 #include <mutex>
+#include <unordered_map>
 
 namespace {
 
@@ -61,6 +67,8 @@ struct SmallArgs {
     int64_t sb, sh, sr;  // K and V share their strides
     float scale;
     int spin_limit;
+    uint32_t *mailbox;    // one word of pinned host memory (device address), or null: receives launch_seq when a wait runs out
+    uint32_t launch_seq;  // never zero
 };
 
 __device__ __forceinline__ void stores_done() {
@@ -78,18 +86,31 @@ __device__ __forceinline__ void st_agent_u64(unsigned long long *p, unsigned lon
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// A bounded wait ran out.  The unit's error word is sticky (only the host's initialisation clears
+// it), the block remembers that its results are void, and the host is told through pinned memory
+// (a system-scope store: this path is never taken in a healthy run).
+constexpr uint32_t kSyncErrBit = 0x80000000u;  // of sync_cnt: a wait of this launch ran out
+__device__ __forceinline__ void give_up(UnitState *st, uint32_t *s_bad, uint32_t *mailbox, uint32_t seq) {
+    dc_st_agent(&st->sync_err, 1u);
+    // also in the arrival counter, where the block that merges finds it in what its own arrival
+    // returns, at no extra memory round trip
+    atomicOr(&st->sync_cnt, kSyncErrBit);
+    __hip_atomic_store(s_bad, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (mailbox) __hip_atomic_store(mailbox, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Every block of the unit has arrived `target` times in all.  Called by all threads.
-__device__ __forceinline__ void unit_barrier(UnitState *st, uint32_t target, int spin_limit) {
+__device__ __forceinline__ void unit_barrier(UnitState *st, uint32_t target, const SmallArgs &a, uint32_t *s_bad) {
     stores_done();
     __syncthreads();
     if (threadIdx.x == 0) {
         atomicAdd(&st->sync_cnt, 1u);
         int spins = 0;
-        while (dc_ld_agent(&st->sync_cnt) < target && spins < spin_limit) {
+        while ((dc_ld_agent(&st->sync_cnt) & ~kSyncErrBit) < target && spins < a.spin_limit) {
             __builtin_amdgcn_s_sleep(1);
             ++spins;
         }
-        if (spins >= spin_limit) dc_st_agent(&st->sync_err, 1u);
+        if (spins >= a.spin_limit) give_up(st, s_bad, a.mailbox, a.launch_seq);
     }
     __syncthreads();
 }
@@ -174,6 +195,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     __shared__ uint32_t s_cnt[4];   // [2]: this block's selected rows so far
     __shared__ uint32_t s_base[2];  // scratch of the radix select
     __shared__ uint32_t s_flag;
+    __shared__ uint32_t s_bad;  // this block's results are void: a wait ran out, here or in an earlier launch
     float *s_scores = reinterpret_cast<float *>(smem);
     unsigned long long *s_cand = reinterpret_cast<unsigned long long *>(smem);
     constexpr int kFirst = small_lds_bytes<HD, G>() - kSmallRows * 4;
@@ -191,9 +213,23 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     const int64_t r1 = r0 + a.rows_per_block < a.n_rows ? r0 + a.rows_per_block : a.n_rows;
     const int n_own = r1 > r0 ? (int)(r1 - r0) : 0;
     const uint32_t bpu = (uint32_t)a.bpu;
+    uint32_t *io = a.idx_out + (int64_t)unit * a.idx_stride;
+    // A unit in which a wait ran out has no valid result: NaN over its output rows and 0xffffffff
+    // over its ids, so that the step cannot pass for a good one downstream.
+    auto poison = [&]() {
+        for (int o = tid; o < G * HD; o += kThreads) a.out[(int64_t)unit * G * HD + o] = 0x7fc0;
+        if (a.lse && tid < G) a.lse[unit * G + tid] = __uint_as_float(0x7fc00000u);
+        for (int i = tid; i < a.k_eff; i += kThreads) io[i] = 0xffffffffu;
+    };
     // ---------------- 1: scores of this block's rows ----------------
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
     if (tid < 4) s_cnt[tid] = 0;
+    // The unit's error word, set by an earlier launch and not cleared since: the shared state
+    // cannot be trusted until the host has initialised it again.  (The load returns while the
+    // rows are scored; it is looked at before the block first touches the shared state.)
+    // A plain load: the word was written by an earlier kernel.
+    uint32_t err0 = 0u;
+    if (tid == 0) err0 = st->sync_err;
     __syncthreads();
     {
         const int grp = lane / LPR, col = lane % LPR;
@@ -227,7 +263,12 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
             }
         }
     }
+    if (tid == 0) s_bad = err0;
     __syncthreads();
+    if (s_bad != 0u) {  // every block of the unit sees the same word: none of them goes on
+        poison();
+        return;
+    }
     // What an addition returns -- the rows of that bucket counted before this block's -- is the
     // block's place among the unit's rows of the bucket: every selected id and every candidate
     // gets its slot from the histogram, and no other counter is needed.
@@ -237,7 +278,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     }
 
     // ---------------- 2: threshold bucket; ids of better buckets, candidates of the threshold bucket ----------------
-    unit_barrier(st, bpu, a.spin_limit);  // the unit's histogram is complete
+    unit_barrier(st, bpu, a, &s_bad);  // the unit's histogram is complete
     uint32_t tb, c_less, n_cand;
     {
         uint32_t bins[kBinsPerThread];
@@ -278,7 +319,6 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     __syncthreads();
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;  // from here on: rows of a bucket placed so far
     __syncthreads();
-    uint32_t *io = a.idx_out + (int64_t)unit * a.idx_stride;
     unsigned long long *cl = a.cand + (int64_t)unit * a.n_rows;
     for (int i = tid; i < n_own; i += kThreads) {
         uint32_t key, bucket;
@@ -318,7 +358,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
                     v8[j] = ld_agent_u64(cl + i);
                     ++spins;
                 }
-                if (v8[j] == kEmpty) dc_st_agent(&st->sync_err, 1u);
+                if (v8[j] == kEmpty) give_up(st, &s_bad, a.mailbox, a.launch_seq);
                 if (i < n_cand) s_cand[i] = v8[j];
             }
         }
@@ -333,8 +373,9 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
         for (uint32_t e0 = 0; e0 < n_oc; e0 += per_pass) {
             const uint32_t e = e0 + (uint32_t)tid / T;
             const uint32_t slot = base_c + e;
-            const bool active = e < n_oc && slot < n_cand;
-            const unsigned long long mine = active ? s_cand[slot] : 0ull;
+            // (a slot that still reads empty after a wait that ran out is nobody's candidate)
+            const unsigned long long mine = (e < n_oc && slot < n_cand) ? s_cand[slot] : kEmpty;
+            const bool active = mine != kEmpty && (uint32_t)mine < (uint32_t)a.n_rows;
             uint32_t rank = 0;
 #pragma unroll 4
             for (uint32_t j = sub; j < n_pair; j += T) {
@@ -352,7 +393,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
         // Too many candidates to rank in LDS (equal keys by the thousand): once every block has
         // written its candidates, block 0 of the unit finds the cutoff, the need-th smallest
         // (key, id) pair, with a radix select over the list.
-        unit_barrier(st, 2u * bpu, a.spin_limit);
+        unit_barrier(st, 2u * bpu, a, &s_bad);
         if (blk == 0) {
             uint32_t *lh = reinterpret_cast<uint32_t *>(smem);  // kRadixBins words
             uint32_t prefix = 0u, rem = need, eq = n_cand;
@@ -424,7 +465,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
                 dc_st_agent(&st->cut_id, t_idx);
             }
         }
-        unit_barrier(st, 3u * bpu, a.spin_limit);
+        unit_barrier(st, 3u * bpu, a, &s_bad);
         arrivals = 3u;
         const uint32_t cut_key = dc_ld_agent(&st->cut_key), cut_id = dc_ld_agent(&st->cut_id);
         for (uint32_t e = tid; e < n_oc; e += kThreads) {
@@ -432,7 +473,7 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
             if (slot >= n_cand) continue;
             const unsigned long long c = ld_agent_u64(cl + slot);
             const uint32_t key = (uint32_t)(c >> 32), id = (uint32_t)c;
-            if (key < cut_key || (key == cut_key && id <= cut_id)) {
+            if (id < (uint32_t)a.n_rows && (key < cut_key || (key == cut_key && id <= cut_id))) {
                 own_win[atomicAdd(&s_cnt[2], 1u)] = id;
                 const uint32_t gs = c_less + atomicAdd(&st->win_cnt, 1u);
                 if (gs < (uint32_t)a.k_eff) io[gs] = id;
@@ -570,7 +611,16 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     __syncthreads();
     if (tid == 0) s_flag = atomicAdd(&st->sync_cnt, 1u);
     __syncthreads();
-    if (s_flag != (arrivals + 1u) * bpu - 1u) return;
+    // A wait that ran out in this launch: the outputs are marked by every block whose own wait ran
+    // out and by the merging block, which finds the error bit of any block that arrived before it
+    // in the counter (a block sets the bit before its next arrival, and counts that do not add up
+    // -- the only way a block could be taken for the last one too early -- come from a wait that
+    // ran out earlier).
+    const bool bad_self = s_bad != 0u;
+    if ((s_flag & ~kSyncErrBit) != (arrivals + 1u) * bpu - 1u) {
+        if (bad_self) poison();
+        return;
+    }
 
     // ---------------- merge of the unit's partials (the last block to arrive) ----------------
     // Every block of the unit is done with the shared state: leave it ready for the next call
@@ -580,6 +630,10 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     if (tid == 0) {
         dc_st_agent(&st->win_cnt, 0u);
         dc_st_agent(&st->sync_cnt, 0u);
+    }
+    if (bad_self || (s_flag & kSyncErrBit) != 0u) {
+        poison();
+        return;
     }
     // Four adjacent output columns per thread, the partials read 16 bytes at a time and a batch
     // of them in flight at once.  With fewer column quads than threads the partials are dealt
@@ -705,9 +759,53 @@ SmallPlan plan_small(int n_units, int region) {
 
 std::atomic<int> g_small_wait_limit{0};  // polls a block's wait may take (0: the default)
 
-// blocks of small_layer_kernel<HD, G> that the device holds at once (0: not asked yet, -1: unknown), per (hd, group)
-int g_small_occ[3][9];
+// What the host keeps per device for this route.
+//   occ       blocks of small_layer_kernel<HD, G> that the device holds at once (0: not asked yet,
+//             -1: unknown), per (hd, group)
+//   last      the stream that the last launch of the kernel outside stream capture went to.  A
+//             call on ANOTHER stream asks whether that stream has run dry (hipStreamQuery: no
+//             wait, nothing enqueued); while it has not, a launch here could overlap with the
+//             last one.  (An event behind every launch would say the same a little more
+//             precisely, but an event is a packet of its own in the queue: 5 us on a 36 us layer.)
+//   mail      one word of pinned, mapped host memory: a block whose wait runs out stores its
+//             launch number there, and the host looks at it (a plain read) at every later call
+constexpr int kMaxDevices = 64;
+struct SmallDev {
+    int occ[3][9];
+    hipStream_t last;
+    bool have;
+    volatile uint32_t *mail_host;
+    uint32_t *mail_dev;
+    bool mail_tried;
+};
+SmallDev g_dev[kMaxDevices];
 std::mutex g_small_mutex;
+uint32_t g_launch_seq = 0;
+// Failures seen so far in this process.  Every workspace remembers the count at which its select
+// state was last initialised; a call on a workspace that lags behind initialises the state
+// again whatever the caller says about it (any workspace may have been the one that failed).
+std::atomic<uint32_t> g_err_epoch{0};
+std::unordered_map<const void *, uint32_t> g_ws_epoch;
+
+// Looks at the mailbox of device `dev` (under g_small_mutex).
+void observe_mailbox(int dev) {
+    SmallDev &d = g_dev[dev];
+    if (!d.mail_host) return;
+    if (*d.mail_host != 0u) {
+        *d.mail_host = 0u;  // a store of the device that lands between the two lines reports a launch that
+                            // was enqueued before anything this observation leads to, so nothing is lost
+        g_err_epoch.fetch_add(1u);
+    }
+}
+
+int current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return dev;
+}
 
 template <int HD, int G>
 int small_occupancy() {
@@ -756,6 +854,45 @@ int launch_small(int group, dim3 grid, hipStream_t st, const SmallArgs &a) {
 
 extern "C" void dc_set_wait_limit(int polls) { g_small_wait_limit.store(polls > 0 ? polls : 0); }
 
+// The rule that keeps two launches of the kernel from overlapping, as a pure function (1: the
+// kernel may be launched now, 0: the call takes the chain of kernels instead).
+extern "C" int dc_one_kernel_guard(int policy, int capturing, int have_prev, int same_stream, int prev_done) {
+    if (policy == DC_ONE_KERNEL_NEVER) return 0;
+    if (policy == DC_ONE_KERNEL_EXCLUSIVE) return 1;  // the caller vouches that nothing else holds CUs
+    if (capturing) return 0;   // a graph is replayed at times and on streams the library never sees
+    if (!have_prev || same_stream) return 1;  // no earlier launch, or the stream orders the two
+    return prev_done ? 1 : 0;
+}
+
+extern "C" unsigned dc_decode_layer_errors(void) {
+    const int dev = current_device();
+    if (dev >= 0) {
+        std::lock_guard<std::mutex> lock(g_small_mutex);
+        observe_mailbox(dev);
+    }
+    return g_err_epoch.load();
+}
+
+// Whether the caller's "the select state is ready" still holds for this workspace: not after a
+// failure that was seen since the state was last initialised.  Looks at the mailbox first.
+bool dc_ws_state_trusted(const void *workspace) {
+    const int dev = current_device();
+    std::lock_guard<std::mutex> lock(g_small_mutex);
+    if (dev >= 0) observe_mailbox(dev);
+    const uint32_t now = g_err_epoch.load();
+    if (now == 0u) return true;  // nothing ever failed: nothing is kept per workspace
+    const auto it = g_ws_epoch.find(workspace);
+    return (it == g_ws_epoch.end() ? 0u : it->second) == now;
+}
+
+// The select state of this workspace is being initialised by the current call.
+void dc_ws_state_initialised(const void *workspace) {
+    const uint32_t now = g_err_epoch.load();
+    if (now == 0u) return;
+    std::lock_guard<std::mutex> lock(g_small_mutex);
+    g_ws_epoch[workspace] = now;
+}
+
 // Whether a layer of these sizes can take the one-kernel route: every block must be resident at
 // once (the blocks of a unit wait for each other), a block's rows must fit its LDS, and the
 // merge must hold the (m, l) pairs of a unit's blocks.
@@ -771,20 +908,21 @@ bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd) {
     const SmallPlan p = plan_small(n_units, region);
     if (!p.ok || p.bpu * group * 2 > kSmallMl) return false;
     const int hi = hd == 64 ? 0 : (hd == 128 ? 1 : 2);
+    const int dev = current_device();
+    if (dev < 0) return false;
     int occ;
     {
         std::lock_guard<std::mutex> lock(g_small_mutex);
-        occ = g_small_occ[hi][group];
-        if (occ == 0) {  // first use: blocks per CU times CUs of the current device
+        occ = g_dev[dev].occ[hi][group];
+        if (occ == 0) {  // first use on this device: blocks per CU times its CUs
             occ = hd == 64 ? small_occupancy_g<64>(group) : (hd == 128 ? small_occupancy_g<128>(group) : small_occupancy_g<256>(group));
-            int dev = 0, cus = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            int cus = 0;
+            if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
                 (void)hipGetLastError();
                 cus = 0;
             }
             occ = occ > 0 && cus > 0 ? occ * cus : -1;
-            g_small_occ[hi][group] = occ;
+            g_dev[dev].occ[hi][group] = occ;
         }
     }
     if (occ <= 0) return false;
@@ -797,6 +935,15 @@ size_t dc_small_workspace_bytes(int n_units, int region, int group, int hd) {
     return carve_attn(nullptr, n_units, group, hd, p.bpu).bytes;
 }
 
+// The route's own candidate lists: one packed (key, id) word per region row.  They are not shared
+// with the lists of the other routes, so a workspace whose state is ready stays ready for this
+// route whichever route the calls in between took.
+size_t dc_small_cand_bytes(int n_units, int region) {
+    const SmallPlan p = plan_small(n_units, region);
+    if (!p.ok) return 0;
+    return dc_align_up((size_t)n_units * (size_t)region * 8, 256);
+}
+
 namespace {
 __global__ void small_list_init_kernel(unsigned long long *list, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -806,20 +953,24 @@ __global__ void small_list_init_kernel(unsigned long long *list, int64_t n) {
 
 // What the one-kernel route needs beyond dc_select_state_init: every slot of the candidate
 // lists empty.  The kernel leaves them so.
-int dc_small_state_init(int n_units, int region, int budget, void *sel_ws, void *stream) {
-    const FusedWs w = carve_fused(sel_ws, n_units, region, budget);
+int dc_small_state_init(int n_units, int region, void *cand, void *stream) {
     const int64_t n = (int64_t)n_units * region;
     if (n <= 0) return DC_OK;
     hipLaunchKernelGGL(small_list_init_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       reinterpret_cast<unsigned long long *>(w.surv), n);
+                       reinterpret_cast<unsigned long long *>(cand), n);
     DC_CHECK_LAUNCH("dc_decode_layer(one kernel, init)");
     return DC_OK;
 }
 
-// The whole layer on `stream`.  sel_ws: the select part of the layer workspace, its state
-// initialised or left ready by the previous call; attn_ws: dc_small_workspace_bytes(...) bytes.
-int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws, void *attn_ws,
-                    size_t attn_ws_bytes, void *stream) {
+// The whole layer on `stream`, unless the launch could overlap with an earlier one of this kernel
+// on another stream (or sits in a graph under capture, whose replays the library never sees): two
+// such launches would each hold part of the CUs and wait for blocks that cannot start.  Returns
+// 1 when the kernel was launched, 0 when the caller has to take the chain of kernels, or a
+// negative DC_E* code.  sel_ws: the select part of the layer workspace, its state initialised or
+// left ready by the previous call; cand: dc_small_cand_bytes(...) bytes, every slot empty;
+// attn_ws: dc_small_workspace_bytes(...) bytes.
+int dc_small_try(const dc_layer_args *a, int region, int k_eff, void *sel_ws, void *cand, void *attn_ws,
+                 size_t attn_ws_bytes, void *stream) {
     const char *who = "dc_decode_layer(one kernel)";
     const int n_units = a->n_b * a->n_h;
     const SmallPlan p = plan_small(n_units, region);
@@ -834,11 +985,56 @@ int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws,
     DC_REQUIRE(a->mode == DC_MODE_IP || a->mode == DC_MODE_REF_DIST, "%s: bad mode %d", who, a->mode);
     DC_REQUIRE(a->idx_unit_stride >= k_eff, "%s: idx_unit_stride < min(budget, region rows)", who);
     DC_REQUIRE(a->recent_lo + a->n_recent < 0xffffffffll, "%s: row numbers out of range", who);
+    DC_REQUIRE(a->one_kernel >= DC_ONE_KERNEL_NEVER && a->one_kernel <= DC_ONE_KERNEL_EXCLUSIVE,
+               "%s: bad one_kernel policy %d", who, a->one_kernel);
     const FusedWs w = carve_fused(sel_ws, n_units, region, a->budget);
     const AttnWs aw = carve_attn(attn_ws, n_units, a->group, a->hd, p.bpu);
     if (attn_ws_bytes < aw.bytes) {
         dc_set_error("%s: workspace %zu bytes < %zu needed", who, attn_ws_bytes, aw.bytes);
         return DC_ENOMEM;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int dev = current_device();
+    DC_REQUIRE(dev >= 0, "%s: no current device (or device number >= %d)", who, kMaxDevices);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusNone;
+    }
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+
+    std::lock_guard<std::mutex> lock(g_small_mutex);
+    SmallDev &d = g_dev[dev];
+    bool prev_done = true;
+    const bool same = d.have && d.last == st;
+    if (a->one_kernel == DC_ONE_KERNEL_AUTO && !capturing && d.have && !same) {
+        // Has the last launch, on the other stream, ended?  (A stream under capture cannot be
+        // asked; a handle that is no longer a stream has nothing in flight that we know of.)
+        prev_done = false;
+        hipStreamCaptureStatus lc = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(d.last, &lc) == hipSuccess && lc == hipStreamCaptureStatusNone) {
+            const hipError_t e = hipStreamQuery(d.last);
+            prev_done = e == hipSuccess;
+            if (e == hipErrorInvalidHandle || e == hipErrorInvalidResourceHandle || e == hipErrorContextIsDestroyed) {
+                d.have = false;
+                prev_done = true;
+            }
+        }
+        (void)hipGetLastError();
+    }
+    if (!dc_one_kernel_guard(a->one_kernel, capturing ? 1 : 0, d.have ? 1 : 0, same ? 1 : 0, prev_done ? 1 : 0))
+        return 0;
+    if (!capturing && !d.mail_tried) {  // (no allocation inside a capture)
+        d.mail_tried = true;
+        void *hp = nullptr, *dp = nullptr;
+        if (hipHostMalloc(&hp, 64, hipHostMallocMapped | hipHostMallocCoherent) == hipSuccess && hp &&
+            hipHostGetDevicePointer(&dp, hp, 0) == hipSuccess && dp) {
+            d.mail_host = static_cast<volatile uint32_t *>(hp);
+            *d.mail_host = 0u;
+            d.mail_dev = static_cast<uint32_t *>(dp);
+        } else {
+            (void)hipGetLastError();  // no mailbox: failures are still marked in the outputs and in the status call
+        }
     }
     SmallArgs s;
     s.Q = (const uint16_t *)a->q;
@@ -848,7 +1044,7 @@ int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws,
     s.new_v = (const uint16_t *)a->new_v;
     s.hist = w.hist;
     s.state = w.state;
-    s.cand = reinterpret_cast<unsigned long long *>(w.surv);
+    s.cand = reinterpret_cast<unsigned long long *>(cand);
     s.idx_out = a->idx_out;
     s.idx_stride = a->idx_unit_stride;
     s.ws_acc = aw.acc;
@@ -869,13 +1065,19 @@ int dc_small_launch(const dc_layer_args *a, int region, int k_eff, void *sel_ws,
     s.sb = a->kv_batch_stride, s.sh = a->kv_head_stride, s.sr = a->kv_row_stride;
     s.scale = a->scale;
     s.spin_limit = g_small_wait_limit.load() > 0 ? g_small_wait_limit.load() : (1 << 20);
+    s.mailbox = d.mail_dev;
+    if (++g_launch_seq == 0u) g_launch_seq = 1u;
+    s.launch_seq = g_launch_seq;
     dim3 grid((unsigned)(n_units * p.bpu));
-    hipStream_t st = (hipStream_t)stream;
     int rc;
     if (a->hd == 64) rc = launch_small<64>(a->group, grid, st, s);
     else if (a->hd == 128) rc = launch_small<128>(a->group, grid, st, s);
     else rc = launch_small<256>(a->group, grid, st, s);
     DC_REQUIRE(rc == 0, "%s: unsupported group %d", who, a->group);
     DC_CHECK_LAUNCH(who);
-    return DC_OK;
+    if (!capturing) {
+        d.last = st;
+        d.have = true;
+    }
+    return 1;
 }

@@ -85,13 +85,22 @@ class DiffCache:
         key_sketch: bool = True,
         use_k_check: bool = False,
         hook_order: int = hip.ORDER_BEST,
+        exclusive_gpu: bool = False,
     ) -> None:
         # hook_order: order of the ids that decode_query_kvcache selects, hence of the rows that
         # decode_post_query_operation gathers into kbuf/vbuf.  ORDER_BEST is the reference's
         # (best first, nsw.rs:592-630); attention over the buffer does not depend on the order, so
         # a caller that only attends may pass hip.ORDER_ANY and save the sort.
+        # exclusive_gpu: the caller vouches that nothing else keeps CUs of this GPU busy while this
+        # cache decodes (no second cache decoding on another stream, no long-lived kernels).  Short
+        # contexts then run as one kernel under graph capture too; without it a captured step takes
+        # the kernel chain, and an eager one does whenever another cache's one-kernel launch is
+        # still in flight on another stream.
         hip.require(hook_order in (hip.ORDER_ANY, hip.ORDER_BEST, hip.ORDER_INDEX), "bad hook_order")
         self.hook_order = hook_order
+        self.one_kernel = hip.ONE_KERNEL_EXCLUSIVE if exclusive_gpu else hip.ONE_KERNEL_AUTO
+        self._errors_seen = hip.decode_layer_errors()
+        self.failed_steps = 0         # decode steps whose one-kernel launch reported a wait that ran out
         self.num_layers = num_layers
         self.batch_size = batch_size
         self.max_length = max_length
@@ -352,6 +361,8 @@ class DiffCache:
         a step; the suffix grows by one after the last layer."""
         b, hq, hkv, hd = self.batch_size, self.num_q_heads, self.num_kv_heads, self.head_dim
         capturing = torch.cuda.is_current_stream_capturing()
+        if layer_idx == 0:
+            self._note_failures()
         if layer_idx == 0 and self.window_full() and not capturing:
             self.rollover()                                                  # diffcache.py:221 asserts instead
         hip.require(self.kvbuf_suffix_len < self.kvbuf_suffix_maxlen,
@@ -382,7 +393,8 @@ class DiffCache:
                              self.kvbuf_suffix_maxlen, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
                              nk, nv, mode=self.mode, order=order,
                              select_state_ready=self._ws_ready and self._ws_order == order,
-                             sketch=self.sketch[layer_idx], n_recent_dev=self.step_state)
+                             sketch=self.sketch[layer_idx], n_recent_dev=self.step_state,
+                             one_kernel=self.one_kernel)
             self._ws_ready = True
             self._ws_order = order      # the state is left ready for a call of the same order only
             self._hook_ws_ready = False
@@ -392,6 +404,20 @@ class DiffCache:
                 self.kvbuf_suffix_len += 1
                 self._store_suffix_rows += 1
         return out
+
+    def _note_failures(self) -> None:
+        """A one-kernel launch of this process reported a wait between its blocks that ran out
+        (read from pinned host memory, no synchronisation): that step's outputs were NaN.  The
+        select state of the workspace is initialised again on the next call, and this cache
+        stays on the kernel chain from here on: whatever starved the kernel of CUs may still be
+        there."""
+        n = hip.decode_layer_errors()
+        if n != self._errors_seen:
+            self.failed_steps += n - self._errors_seen
+            self._errors_seen = n
+            self._ws_ready = False
+            self._hook_ws_ready = False
+            self.one_kernel = hip.ONE_KERNEL_NEVER
 
     def _decode_attention_k_check(self, layer_idx: int, q: torch.Tensor, nk: torch.Tensor, nv: torch.Tensor,
                                   out: torch.Tensor, ws: torch.Tensor) -> None:

@@ -330,8 +330,8 @@ typedef struct dc_layer_args {
                              initialised first.  1: the caller vouches that the last call on this
                              workspace was a dc_decode_layer with the same n_b, n_h, group, hd,
                              region length, budget and order and scores == NULL (with or without
-                             a sketch), which leaves the select state ready; the init kernels
-                             are skipped */
+                             a sketch, whichever route it took), which leaves the select state
+                             ready; the init kernels are skipped */
     void *ev_scan_begin;  /* optional hipEvent_t pair recorded on `stream` right before and */
     void *ev_scan_end;    /* right after the scan kernel (for timing it in place), or NULL */
     const uint8_t *sketch_codes; /* NULL, or the sketch of the K store (row 0 = store row 0): the
@@ -342,6 +342,8 @@ typedef struct dc_layer_args {
     int64_t sketch_batch_stride, sketch_head_stride, sketch_row_stride; /* bytes */
     const int32_t *n_recent_dev; /* NULL, or the device-side length of the suffix (see
                              dc_gather_attn_bf16): n_recent is then its capacity */
+    int one_kernel;       /* a DC_ONE_KERNEL_* value: when a short context may run as one kernel
+                             (see "Short contexts" below); 0 = DC_ONE_KERNEL_AUTO */
 } dc_layer_args;
 
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,
@@ -350,20 +352,51 @@ int dc_decode_layer(const dc_layer_args *args, void *stream);
 /*
  * Short contexts.  With scores == NULL, order == DC_ORDER_ANY and at most 640 Ki region rows
  * over all units, dc_decode_layer runs the layer as ONE kernel whose blocks are all resident
- * and hand their phases over through the workspace (same results; the event pair then brackets
- * that kernel).  Its waits between blocks are bounded; dc_decode_layer_status waits for
- * `stream` and returns DC_EDEVICE if a wait of the last calls on this workspace ran out (never
- * observed; the outputs would be invalid), DC_OK otherwise.  `args` as in the call it checks.
- * The kernel counts on all its blocks running at the same time (two per CU): it may share the
- * GPU with short kernels of other streams, which only delay it, but not with kernels that keep
- * CUs occupied for good -- then its waits run out (after about a second each) instead of ending.
+ * (two per CU) and hand their phases over through the workspace (same results; the event pair
+ * then brackets that kernel).  No counterpart in the reference, whose layers run on the CPU pool
+ * (lib.rs:352-369); what it has to match is that one layer call is always right
+ * (src/diffcache/base.py:150-155).
+ *
+ * The kernel counts on all its blocks running at the same time.  It may share the GPU with
+ * short kernels of other streams, which only delay it, but not with a second launch of itself
+ * on another stream (two DiffCache objects, two sequences decoded side by side: each launch
+ * would get part of the CUs and wait for blocks that cannot start), nor with kernels that keep
+ * CUs occupied for good.  What the library does about it:
+ *   - it remembers, per device, the stream of the last launch of the kernel; a dc_decode_layer
+ *     on ANOTHER stream while that stream still has work in flight (hipStreamQuery, never a
+ *     wait) takes the chain of kernels of the long contexts instead (same ids, same attention
+ *     within rounding).
+ *     A call on a stream that is being captured takes the chain too, because a graph is replayed
+ *     at times the library never sees.  dc_layer_args.one_kernel overrides this:
+ *     DC_ONE_KERNEL_EXCLUSIVE: the caller vouches that no other launch of the kernel and no
+ *     long-lived kernel shares the GPU (the kernel is then launched under capture as well);
+ *     DC_ONE_KERNEL_NEVER: always the chain.  dc_last_route() says what the last call took;
+ *   - the waits between blocks are bounded (about a second each).  If one runs out all the
+ *     same, the call's results are void and say so: the out rows (and lse) of the unit are NaN
+ *     and its ids 0xffffffff (do not gather with them), the unit's error word in the workspace
+ *     stays set, and every later one-kernel call on that workspace returns NaN as well until the
+ *     select state is initialised again;
+ *   - it initialises that state again by itself: the failing kernel also stores into a word of
+ *     pinned host memory, which every dc_decode_layer call reads (no copy, no wait); from then
+ *     on the first call on every workspace ignores select_state_ready == 1 once.  Calls that
+ *     were enqueued before the failure was seen return NaN; a captured graph cannot be mended
+ *     this way (its launches are fixed): capture it again, or take it out of use, when
+ *     dc_decode_layer_errors() has moved.
+ * dc_decode_layer_errors: the number of failures seen so far in this process (reads the
+ * pinned word of the current device, waits for nothing).
+ * dc_decode_layer_status waits for `stream` and returns DC_EDEVICE if the error word of a unit
+ * of this workspace is set, DC_OK otherwise.  `args` as in the call it checks.
  * DIFFCACHE_ONE_KERNEL=0 in the environment of the process switches the route off.
- * No counterpart in the reference, whose layers run on the CPU pool (lib.rs:352-369).
  */
+#define DC_ONE_KERNEL_AUTO 0
+#define DC_ONE_KERNEL_EXCLUSIVE 1
+#define DC_ONE_KERNEL_NEVER (-1)
 int dc_decode_layer_status(const dc_layer_args *args, void *stream);
+unsigned dc_decode_layer_errors(void);
 /*
- * Which kernels a dc_decode_layer call with these arguments runs (pointers are not followed):
- * a DC_ROUTE_* value, or a negative DC_E* code.
+ * Which kernels a dc_decode_layer call with these arguments runs when no other launch of the
+ * one-kernel route is in the way (pointers are not followed): a DC_ROUTE_* value, or a negative
+ * DC_E* code.  dc_last_route: the route that the last dc_decode_layer call of this thread took.
  */
 #define DC_ROUTE_ATTEND_ONLY 0 /* nothing to select (empty region or budget 0) */
 #define DC_ROUTE_DENSE 1       /* fp32 scores materialised: dc_score_bf16 + dc_topk_select */
@@ -371,11 +404,19 @@ int dc_decode_layer_status(const dc_layer_args *args, void *stream);
 #define DC_ROUTE_SKETCH 3      /* dc_score_select_sketch_bf16 */
 #define DC_ROUTE_ONE_KERNEL 4  /* short context: the whole layer in one kernel */
 int dc_decode_layer_route(const dc_layer_args *args);
+int dc_last_route(void);
+/*
+ * The rule by which a call is kept off the one-kernel route, as a function of what the library
+ * knows at the call (exposed so that the rule can be tested without a GPU): 1 = launch the
+ * kernel, 0 = take the chain.  policy: dc_layer_args.one_kernel; capturing: the stream is under
+ * capture; have_prev: the kernel was launched on this device before; same_stream: on this very
+ * stream; prev_done: that launch's stream has nothing in flight any more.
+ */
+int dc_one_kernel_guard(int policy, int capturing, int have_prev, int same_stream, int prev_done);
 /*
  * For tests of that error path: the number of polls after which a block of the one-kernel
  * route gives up a wait (0: the default, about a second).  With a tiny limit the kernel still
- * runs to its end, its outputs are not valid, dc_decode_layer_status reports DC_EDEVICE and the
- * next call on the workspace needs select_state_ready == 0.  Process-wide.
+ * runs to its end and behaves as described above for a wait that ran out.  Process-wide.
  */
 void dc_set_wait_limit(int polls);
 

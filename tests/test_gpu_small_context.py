@@ -147,8 +147,11 @@ def test_small_context_benchmark_shape_with_a_device_side_window():
 
 
 def test_small_context_bounded_wait_is_reported():
-    """With a wait limit of one poll the blocks give up their waits: the kernel still ends, the
-    status call reports it, and after a fresh initialisation the route works again."""
+    """With a wait limit of one poll the blocks give up their waits.  The kernel still ends; the
+    step cannot pass for a good one (NaN outputs, ids 0xffffffff); the host learns of it without
+    a synchronising call (dc_decode_layer_errors); later calls on the workspace return NaN as long
+    as the state is not initialised again; and the library initialises it again by itself on the
+    next call, although that call says select_state_ready."""
     rng = np.random.default_rng(304)
     b, hq, hkv, hd, n_ctx = 1, 8, 2, 128, 30000
     k, v = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd)
@@ -157,16 +160,190 @@ def test_small_context_bounded_wait_is_reported():
     p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
     ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, 512, hq // hkv, hd, 512 + 4 + 64 + 1), DEV)
     idx = torch.zeros((b * hkv, 512), dtype=torch.int32, device=DEV)
-    out = torch.empty((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    lse = torch.zeros((b, hq), dtype=torch.float32, device=DEV)
     args = (qd, kd, vd, p_len, hi, s_len, 512, None, idx, out, ws)
+    errors0 = hip.decode_layer_errors()
     hip.lib.dc_set_wait_limit(1)
     try:
-        hip.decode_layer(*args, order=hip.ORDER_ANY)
+        print("forced give-up: one-kernel launch with a wait limit of one poll", flush=True)
+        hip.decode_layer(*args, lse=lse, order=hip.ORDER_ANY)
+        assert hip.last_route() == hip.ROUTE_ONE_KERNEL
         with pytest.raises(hip.DiffCacheError, match="bounded wait"):
             hip.decode_layer_status(*args, order=hip.ORDER_ANY)
     finally:
         hip.lib.dc_set_wait_limit(0)
+    bad_units = [u for u in range(b * hkv) if (idx[u] == -1).all()]
+    assert bad_units, "no unit reported its failure in the ids"
+    g = hq // hkv
+    for u in bad_units:
+        assert torch.isnan(out.view(b * hkv, g, hd)[u].float()).all()
+        assert torch.isnan(lse.view(b * hkv, g)[u]).all()
+    for u in range(b * hkv):        # a unit is either marked as a whole or not at all in its output
+        o = torch.isnan(out.view(b * hkv, g, hd)[u].float())
+        assert o.all() or not o.any()
+    assert hip.decode_layer_errors() > errors0              # read from pinned host memory, no stream wait
+    # with the default limit again, on a second workspace nothing is wrong
+    run_case(k, v, q, None, None, n_ctx, 512, 4, 64, orc.MODE_REF_DIST, reps=2)
+    # the workspace of the failed call: the caller still says "ready"; the library knows better
+    print("forced give-up: next call on the same workspace, select_state_ready=1", flush=True)
+    idx.fill_(7)
+    out.zero_()
+    hip.decode_layer(*args, order=hip.ORDER_ANY, select_state_ready=True)
+    assert hip.last_route() == hip.ROUTE_ONE_KERNEL
+    hip.decode_layer_status(*args, order=hip.ORDER_ANY)     # the error words are clear again
+    assert not torch.isnan(out.float()).any()
+    dense = hip.score(kd, qd, lo, hi - lo, orc.MODE_REF_DIST, q_group=g).cpu().numpy()
+    ids = idx.cpu().numpy().astype(np.int64)
+    for u in range(b * hkv):
+        want = orc.topk_select(dense[u], 512, orc.MODE_REF_DIST).astype(np.int64)
+        assert np.array_equal(np.sort(ids[u]), np.sort(want)), u
     run_case(k, v, q, None, None, n_ctx, 512, 4, 64, orc.MODE_REF_DIST, reps=2, ws=ws)
+
+
+def test_small_context_sticky_error_marks_later_calls_until_initialised():
+    """A captured graph cannot be mended by the library (its launches are fixed).  What it must
+    not do is return stale numbers: with the unit's error word set, every later one-kernel launch
+    on the workspace marks its outputs, until the state is initialised again."""
+    rng = np.random.default_rng(307)
+    b, hq, hkv, hd, n_ctx = 1, 8, 2, 128, 9000
+    k, v, q = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hq, hd)
+    kd, vd, qd = to_dev_bf16(k), to_dev_bf16(v), to_dev_bf16(q)
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+    ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, 256, hq // hkv, hd, 256 + 69), DEV)
+    idx = torch.zeros((b * hkv, 256), dtype=torch.int32, device=DEV)
+    out = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+    args = (qd, kd, vd, p_len, hi, s_len, 256, None, idx, out, ws)
+    # two calls enqueued back to back, the second before the host can have seen the first fail
+    hip.lib.dc_set_wait_limit(1)
+    try:
+        print("sticky error: failing launch, then a launch enqueued behind it", flush=True)
+        hip.decode_layer(*args, order=hip.ORDER_ANY)
+    finally:
+        hip.lib.dc_set_wait_limit(0)
+    out2 = torch.zeros_like(out)
+    idx2 = torch.zeros_like(idx)
+    args2 = (qd, kd, vd, p_len, hi, s_len, 256, None, idx2, out2, ws)
+    # (the error count is not asked in between: nothing on the host has looked at the mailbox yet
+    #  unless this call does, in which case it initialises the state and the result is good)
+    hip.decode_layer(*args2, order=hip.ORDER_ANY, select_state_ready=True)
+    torch.cuda.synchronize()
+    first_bad = torch.isnan(out.float()).any().item()
+    assert first_bad
+    healed = not torch.isnan(out2.float()).any().item()
+    if healed:      # the host saw the failure in time: the second call must then be right
+        dense = hip.score(kd, qd, lo, hi - lo, orc.MODE_REF_DIST, q_group=hq // hkv).cpu().numpy()
+        for u in range(b * hkv):
+            want = orc.topk_select(dense[u], 256, orc.MODE_REF_DIST).astype(np.int64)
+            assert np.array_equal(np.sort(idx2[u].cpu().numpy().astype(np.int64)), np.sort(want)), u
+    else:           # it did not: every unit whose error word was set is marked, none is stale
+        g = hq // hkv
+        for u in range(b * hkv):
+            if torch.isnan(out.view(b * hkv, g, hd)[u].float()).any():
+                assert torch.isnan(out2.view(b * hkv, g, hd)[u].float()).all(), u
+                assert (idx2[u] == -1).all(), u
+    run_case(k, v, q, None, None, n_ctx, 256, 4, 64, orc.MODE_REF_DIST, reps=2, ws=ws)
+
+
+def test_two_streams_never_run_the_one_kernel_route_side_by_side():
+    """Two sequences decoded on two streams of one process.  While the one-kernel launch of the
+    first is still in flight, a call on the second stream takes the kernel chain (two launches of
+    the kernel would starve each other of CUs); both calls are right.  Once the first has ended,
+    the second stream gets the kernel again."""
+    rng = np.random.default_rng(308)
+    b, hq, hkv, hd, n_ctx, budget = 1, 8, 2, 128, 20000, 384
+    g = hq // hkv
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+    seqs = []
+    for _ in range(2):
+        k, v, q = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hq, hd)
+        kd, vd, qd = to_dev_bf16(k), to_dev_bf16(v), to_dev_bf16(q)
+        sk = hip.Sketch(kd).build(kd, lo, hi - lo)
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, budget, g, hd, budget + 69), DEV)
+        idx = torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV)
+        out = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+        seqs.append(dict(k=k, v=v, q=q, kd=kd, vd=vd, qd=qd, sk=sk, ws=ws, idx=idx, out=out))
+    torch.cuda.synchronize()
+    s_a, s_b = torch.cuda.Stream(), torch.cuda.Stream()
+    big = torch.randn((8192, 8192), device=DEV, dtype=torch.bfloat16)
+    big = (big @ big).clamp_(-1, 1)         # (the GEMM library loads its kernels on first use)
+    torch.cuda.synchronize()
+    routes = []
+
+    def call(sq, sketch):
+        hip.decode_layer(sq["qd"], sq["kd"], sq["vd"], p_len, hi, s_len, budget, None, sq["idx"], sq["out"],
+                         sq["ws"], order=hip.ORDER_ANY, sketch=sq["sk"] if sketch else None)
+        routes.append(hip.last_route())
+
+    print("two streams: stream A busy, one-kernel launch queued behind it; stream B calls meanwhile", flush=True)
+    with torch.cuda.stream(s_a):
+        for _ in range(40):                 # tens of milliseconds of work in front of A's call
+            big = (big @ big).clamp_(-1, 1)
+        call(seqs[0], sketch=True)
+    with torch.cuda.stream(s_b):
+        call(seqs[1], sketch=True)          # A's kernel has not even started: B must not launch a second one
+        call(seqs[1], sketch=False)         # still pending
+    torch.cuda.synchronize()
+    assert routes == [hip.ROUTE_ONE_KERNEL, hip.ROUTE_SKETCH, hip.ROUTE_STREAM], routes
+    with torch.cuda.stream(s_b):
+        call(seqs[1], sketch=True)          # nothing of A is in flight any more
+    torch.cuda.synchronize()
+    assert routes[-1] == hip.ROUTE_ONE_KERNEL
+    for sq in seqs:
+        dense = hip.score(sq["kd"], sq["qd"], lo, hi - lo, orc.MODE_REF_DIST, q_group=g).cpu().numpy()
+        ids = sq["idx"].cpu().numpy().astype(np.int64)
+        got = orc.bf16_to_f32(to_np_u16(sq["out"]))
+        for u in range(b * hkv):
+            bi, h = divmod(u, hkv)
+            want = orc.topk_select(dense[u], budget, orc.MODE_REF_DIST).astype(np.int64)
+            assert np.array_equal(np.sort(ids[u]), np.sort(want)), u
+            rows = np.concatenate([want + lo, np.arange(p_len), np.arange(hi, hi + s_len)]).astype(np.int64)
+            o, _ = orc.sparse_attention(sq["q"][bi, h * g:(h + 1) * g], sq["k"][bi, h][rows], sq["v"][bi, h][rows],
+                                        None, None)
+            assert bf16_close(got[bi, h * g:(h + 1) * g], o), u
+
+
+def test_one_kernel_route_under_capture_needs_the_callers_word():
+    """A stream under capture: the call takes the kernel chain unless the caller vouches for an
+    exclusive GPU (ONE_KERNEL_EXCLUSIVE); replays of both graphs equal the eager result, with eager
+    work and synchronisation between the replays."""
+    rng = np.random.default_rng(309)
+    b, hq, hkv, hd, n_ctx, budget = 1, 8, 2, 128, 12000, 256
+    g = hq // hkv
+    p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+    k, v = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd)
+    kd, vd = to_dev_bf16(k), to_dev_bf16(v)
+    qd = to_dev_bf16(rand_bf16(rng, b, hq, hd))
+    res = {}
+    for policy in (hip.ONE_KERNEL_AUTO, hip.ONE_KERNEL_EXCLUSIVE):
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, budget, g, hd, budget + 69), DEV)
+        idx = torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV)
+        out = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):       # every kernel once outside capture; leaves the state ready
+            hip.decode_layer(qd, kd, vd, p_len, hi, s_len, budget, None, idx, out, ws, order=hip.ORDER_ANY,
+                             one_kernel=policy)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            hip.decode_layer(qd, kd, vd, p_len, hi, s_len, budget, None, idx, out, ws, order=hip.ORDER_ANY,
+                             select_state_ready=True, one_kernel=policy)
+            route = hip.last_route()
+        assert route == (hip.ROUTE_ONE_KERNEL if policy == hip.ONE_KERNEL_EXCLUSIVE else hip.ROUTE_STREAM)
+        res[policy] = (graph, idx, out, ws)
+    for rep in range(3):
+        qd.copy_(to_dev_bf16(rand_bf16(rng, b, hq, hd)))
+        idx_e = torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV)
+        out_e = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+        ws_e = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, budget, g, hd, budget + 69), DEV)
+        hip.decode_layer(qd, kd, vd, p_len, hi, s_len, budget, None, idx_e, out_e, ws_e, order=hip.ORDER_ANY,
+                         one_kernel=hip.ONE_KERNEL_NEVER)
+        torch.cuda.synchronize()
+        for policy, (graph, idx, out, ws) in res.items():
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(torch.sort(idx, dim=1).values, torch.sort(idx_e, dim=1).values), (rep, policy)
+            assert torch.allclose(out.float(), out_e.float(), atol=4e-3, rtol=2.0 ** -6), (rep, policy)
 
 
 def test_prepared_layer_call_equals_decode_layer():

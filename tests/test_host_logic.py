@@ -44,6 +44,27 @@ def test_layer_args_struct_matches_header_order():
     assert names == [f[0] for f in _hip.LayerArgs._fields_]
 
 
+def test_one_kernel_guard_rule():
+    """When a short-context call may run as one kernel (all its blocks wait for each other, so two
+    launches must never overlap): the rule of dc_one_kernel_guard, every combination."""
+    from diffcache_amd import _hip
+    g = _hip.lib.dc_one_kernel_guard
+    auto, excl, never = _hip.ONE_KERNEL_AUTO, _hip.ONE_KERNEL_EXCLUSIVE, _hip.ONE_KERNEL_NEVER
+    for capturing in (0, 1):
+        for have_prev in (0, 1):
+            for same in (0, 1):
+                for done in (0, 1):
+                    assert g(never, capturing, have_prev, same, done) == 0
+                    assert g(excl, capturing, have_prev, same, done) == 1
+                    want = 0 if capturing else int((not have_prev) or same or done)
+                    assert g(auto, capturing, have_prev, same, done) == want, (capturing, have_prev, same, done)
+    # the case the rule exists for: an earlier launch on another stream that has not finished
+    assert g(auto, 0, 1, 0, 0) == 0
+    # no GPU here: nothing has failed, and asking costs nothing
+    assert _hip.decode_layer_errors() == 0
+    assert _hip.last_route() == _hip.ROUTE_ATTEND_ONLY
+
+
 def test_wrappers_refuse_cpu_tensors():
     from diffcache_amd import _hip
     k = torch.zeros((1, 1, 16, 128), dtype=torch.bfloat16)
