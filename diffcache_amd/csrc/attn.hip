@@ -15,6 +15,7 @@
 // the device-scope fence it needs costs far more than a second launch here.)
 // Bound by HBM: 2 * HD*2 bytes per row.
 #include "dc_attn.h"
+#include <cstdlib>
 #include <mutex>
 
 namespace {
@@ -29,6 +30,14 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(AttnArgs a) {
     sh.l = s_mem + kAttnWaves * G;
     sh.acc = s_mem + 2 * kAttnWaves * G;
     dc_attn_split<HD, G>(a, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, sh);
+}
+
+// The same split on the matrix cores (dc_attn_split_mfma); the group is a run-time value here
+// because the products are padded to 16 heads anyway.
+template <int HD>
+__global__ __launch_bounds__(kThreads) void gather_attn_mfma_kernel(AttnArgs a, int group) {
+    extern __shared__ float s_dyn[];
+    dc_attn_split_mfma<HD>(a, group, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, s_dyn);
 }
 
 // out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block
@@ -133,9 +142,27 @@ int launch_attn(int group, dim3 grid, hipStream_t st, const AttnArgs &a) {
 
 }  // namespace
 
+// Which split body a call runs.  The matrix-core version takes any group up to 16; the VALU
+// version (groups up to 8) stays for comparison: DIFFCACHE_ATTN_VALU=1 in the environment of the
+// process (read once) selects it wherever it applies.
+static bool attn_use_mfma(int group, int64_t max_row, int64_t ksr, int64_t vsr) {
+    static const bool valu = [] {
+        const char *e = std::getenv("DIFFCACHE_ATTN_VALU");
+        return e && e[0] == '1' && e[1] == 0;
+    }();
+    if (group > 8) return true;
+    if (valu) return false;
+    // rows are addressed with 32-bit byte offsets from the unit's first row
+    const int64_t sr = ksr > vsr ? ksr : vsr;
+    return (max_row + 1) * sr * 2 <= 0xffffffffll;
+}
+
 extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_rows_attended) {
     if (n_units <= 0 || group <= 0 || hd < 8) return 256;
-    return carve_attn(nullptr, n_units, group, hd, plan_attn(hd, group, n_rows_attended).n_splits).bytes;
+    // room for either split body (the slices of the VALU version are shorter for large groups)
+    const size_t a = carve_attn(nullptr, n_units, group, hd, plan_attn(hd, group, n_rows_attended, false).n_splits).bytes;
+    const size_t b = carve_attn(nullptr, n_units, group, hd, plan_attn(hd, group, n_rows_attended, true).n_splits).bytes;
+    return a > b ? a : b;
 }
 
 namespace {
@@ -155,7 +182,7 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     DC_REQUIRE(n_idx == 0 || idx, "%s: idx is null but n_idx > 0", who);
     DC_REQUIRE((new_k == nullptr) == (new_v == nullptr),
                "%s: new_k and new_v must both be set or both be null", who);
-    DC_REQUIRE(group >= 1 && group <= 8, "%s: group %d not in [1,8]", who, group);
+    DC_REQUIRE(group >= 1 && group <= kMfmaMaxGroup, "%s: group %d not in [1,%d]", who, group, kMfmaMaxGroup);
     DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d unsupported", who, hd);
     DC_REQUIRE(dc_aligned16(k) && dc_aligned16(v) && dc_aligned16(q) &&
                    (!new_k || (dc_aligned16(new_k) && dc_aligned16(new_v))),
@@ -171,7 +198,9 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     const int n_total = n_idx + n_sink + n_recent + (new_k ? 1 : 0);
     DC_REQUIRE(workspace && (((uintptr_t)workspace) & 255u) == 0,
                "%s: workspace must be non-null and 256-byte aligned", who);
-    const AttnPlan plan = plan_attn(hd, group, n_total);
+    const bool mfma = attn_use_mfma(group, recent_lo + n_recent, ksr, vsr);
+    DC_REQUIRE(mfma || group <= 8, "%s: group %d needs rows within 4 GiB of the unit's first row", who, group);
+    const AttnPlan plan = plan_attn(hd, group, n_total, mfma);
     const AttnWs w = carve_attn(workspace, n_units, group, hd, plan.n_splits);
     if (workspace_bytes < w.bytes) {
         dc_set_error("%s: workspace %zu bytes < %zu needed", who, workspace_bytes, w.bytes);
@@ -203,8 +232,13 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     aa.ksb = ksb, aa.ksh = ksh, aa.ksr = ksr, aa.vsb = vsb, aa.vsh = vsh, aa.vsr = vsr;
     aa.scale = scale;
     uint16_t *o16 = (uint16_t *)out;
-    int rc;
-    if (hd == 64) rc = launch_attn<64>(group, grid, st, aa);
+    int rc = 0;
+    if (mfma) {
+        const size_t lds = mfma_shared_bytes(hd, group);
+        if (hd == 64) hipLaunchKernelGGL(gather_attn_mfma_kernel<64>, grid, dim3(kThreads), lds, st, aa, group);
+        else if (hd == 128) hipLaunchKernelGGL(gather_attn_mfma_kernel<128>, grid, dim3(kThreads), lds, st, aa, group);
+        else hipLaunchKernelGGL(gather_attn_mfma_kernel<256>, grid, dim3(kThreads), lds, st, aa, group);
+    } else if (hd == 64) rc = launch_attn<64>(group, grid, st, aa);
     else if (hd == 128) rc = launch_attn<128>(group, grid, st, aa);
     else rc = launch_attn<256>(group, grid, st, aa);
     DC_REQUIRE(rc == 0, "%s: unsupported group %d", who, group);
@@ -250,7 +284,7 @@ extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const vo
                                           const int32_t *n_recent_dev, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh,
                                           int64_t vsr, float scale, void *stream) {
     const char *who = "dc_gather_attn_static_bf16";
-    DC_REQUIRE(n_b >= 0 && n_h >= 1 && group >= 1 && group <= 8 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
+    DC_REQUIRE(n_b >= 0 && n_h >= 1 && group >= 1 && group <= kMfmaMaxGroup && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
                "%s: bad sizes", who);
     DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d unsupported", who, hd);
     const int64_t n_units = (int64_t)n_b * n_h;

@@ -539,7 +539,7 @@ def test_gather_rows_and_ingest_append():
 
 # ------------------------------------------------------------------ attention
 
-@pytest.mark.parametrize("hd,g", [(128, 4), (128, 7), (64, 8), (256, 1), (128, 1)])
+@pytest.mark.parametrize("hd,g", [(128, 4), (128, 7), (64, 8), (256, 1), (128, 1), (128, 16), (64, 12), (256, 9)])
 @pytest.mark.parametrize("n_idx,n_sink,n_recent,new_tok", [(0, 0, 1, False), (5, 0, 0, True),
                                                            (300, 4, 64, True), (1024, 128, 129, False)])
 def test_gather_attention_matches_float64(hd, g, n_idx, n_sink, n_recent, new_tok):
