@@ -10,13 +10,16 @@ constexpr int kRadixBins = 1 << kRadixBits;
 constexpr int kScanBatch = 8;  // items of a list that a thread fetches before it looks at any
 constexpr int kScanShort = 8192;  // lists up to this length sit in LDS (kCandLds of the callers): plain loops
 
-// inclusive scan over the lanes of a wave
-__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        uint32_t t = __shfl_up(v, d, 64);
-        if (lane >= d) v += t;
-    }
+// inclusive scan over the lanes of a wave: four shifts inside the rows of 16 lanes, then the
+// last lane of row 0 (2) is added to row 1 (3), and the last lane of row 1 to rows 2 and 3
+// (data-parallel primitives on the ALU; a shuffle through the LDS crossbar per step costs more)
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, true);   // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, true);   // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, true);   // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, true);   // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
     return v;
 }
 
@@ -40,6 +43,47 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wtot, 
     __syncthreads();
     *total = tot;
     return off + incl - v;
+}
+
+// Slots of a list in LDS for the lanes of a wave that ask for one: one addition per wave instead
+// of one per lane (additions of a whole wave to one LDS word are served one after the other).
+// Must be called by all lanes of the wave; returns the slot of a lane with `want`.
+__device__ __forceinline__ uint32_t wave_reserve(bool want, uint32_t *counter) {
+    const unsigned long long mask = __ballot(want);
+    if (mask == 0ull) return 0u;
+    const int lane = threadIdx.x & 63, leader = (int)__builtin_ctzll(mask);
+    uint32_t base = 0u;
+    if (lane == leader) base = atomicAdd(counter, (uint32_t)__popcll(mask));
+    base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
+    return base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+}
+
+// f(key, id, valid) for every entry of a (key, id) list, by ALL threads the same number of times
+// (valid: the thread has an entry this time), so that f may use wave-wide operations.
+template <int NT, typename F>
+__device__ __forceinline__ void dc_for_each_pair_uniform(const uint32_t *ck, const uint32_t *ci, uint32_t n, F f) {
+    if (n <= (uint32_t)kScanShort) {
+        for (uint32_t i0 = 0; i0 < n; i0 += NT) {
+            const uint32_t i = i0 + threadIdx.x;
+            const bool in = i < n;
+            f(in ? ck[i] : 0u, in ? ci[i] : 0u, in);
+        }
+        return;
+    }
+    for (uint32_t i0 = 0; i0 < n; i0 += kScanBatch * NT) {
+        uint32_t key[kScanBatch], id[kScanBatch];
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) {
+            const uint32_t i = i0 + (uint32_t)u * NT + threadIdx.x;
+            key[u] = id[u] = 0u;
+            if (i < n) {
+                key[u] = ck[i];
+                id[u] = ci[i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kScanBatch; ++u) f(key[u], id[u], i0 + (uint32_t)u * NT + threadIdx.x < n);
+    }
 }
 
 // f(key, id) for every entry of a (key, id) list, kScanBatch entries of a thread in flight.
@@ -144,7 +188,7 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
 // threshold value; *rem_out = how many items equal to it are needed (rank of the
 // threshold inside its tie group), *n_eq = size of the tie group.
 template <typename Get>
-__device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int top, uint32_t prefix,
+__device__ __forceinline__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int top, uint32_t prefix,
                                        uint32_t eq, uint32_t *lh, uint32_t *wtot, uint32_t *sres,
                                        uint32_t *rem_out, uint32_t *n_eq) {
     while (top > 0) block_radix_pass(get, n, prefix, rem, eq, top, lh, wtot, sres);
@@ -158,7 +202,7 @@ __device__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int to
 // block with uniform arguments.  lh: kRadixBins words, wtot: kFinalThreads/64+1
 // words, sres: 4 words, smisc: 2 words of LDS.  kout (optional) receives the
 // key of each id written.
-__device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_t n_c, uint32_t need,
+__device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_t n_c, uint32_t need,
                                  uint32_t *io, int n_rows, uint32_t *lh, uint32_t *wtot,
                                  uint32_t *sres, uint32_t *smisc, uint32_t *kout = nullptr) {
     const int tid = threadIdx.x;
@@ -190,7 +234,10 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
 #pragma unroll
         for (int u = 0; u < kScanBatch; ++u) diff |= v[u] ^ k0;
     }
-    if (diff) atomicOr(&smisc[0], diff);
+    // one addition per wave: a thousand lanes updating one LDS word are served one after the other
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) diff |= (uint32_t)__shfl_xor((int)diff, d, 64);
+    if ((tid & 63) == 0 && diff) atomicOr(&smisc[0], diff);
     __syncthreads();
     diff = smisc[0];
     const int hb = diff ? 31 - __clz(diff) : -1;
@@ -213,18 +260,16 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
         __syncthreads();
         const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
         const uint32_t base = need - rem;  // members from the bins below the threshold bin
-        dc_for_each_pair<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id) {
+        dc_for_each_pair_uniform<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
             const uint32_t hi = key & himask, ph = prefix & himask;
-            if (hi < ph) {
-                const uint32_t slot = atomicAdd(&smisc[1], 1u);
-                if (slot < base) {
-                    io[slot] = id;
-                    if (kout) kout[slot] = key;
-                }
-            } else if (hi == ph) {
-                const uint32_t e = atomicAdd(&smisc[0], 1u);
-                if (e < (uint32_t)kFinalThreads) tie[e] = ((unsigned long long)key << 32) | id;
+            const bool member = in && hi < ph, tied = in && hi == ph;
+            const uint32_t slot = wave_reserve(member, &smisc[1]);
+            if (member && slot < base) {
+                io[slot] = id;
+                if (kout) kout[slot] = key;
             }
+            const uint32_t e = wave_reserve(tied, &smisc[0]);
+            if (tied && e < (uint32_t)kFinalThreads) tie[e] = ((unsigned long long)key << 32) | id;
         });
         __syncthreads();
         const uint32_t n_t = smisc[0] < (uint32_t)kFinalThreads ? smisc[0] : (uint32_t)kFinalThreads;
@@ -256,13 +301,12 @@ __device__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_
         t_idx = block_radix_select(get_idx, n_c, need_eq, hbi + 1, 0u, n_eq, lh, wtot, sres, &r2, &e2);
     }
 
-    dc_for_each_pair<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id) {
-        if (key < t_key || (key == t_key && id <= t_idx)) {
-            uint32_t slot = atomicAdd(&smisc[1], 1u);
-            if (slot < need) {
-                io[slot] = id;
-                if (kout) kout[slot] = key;
-            }
+    dc_for_each_pair_uniform<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
+        const bool member = in && (key < t_key || (key == t_key && id <= t_idx));
+        const uint32_t slot = wave_reserve(member, &smisc[1]);
+        if (member && slot < need) {
+            io[slot] = id;
+            if (kout) kout[slot] = key;
         }
     });
 }

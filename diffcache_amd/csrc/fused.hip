@@ -810,11 +810,18 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     UnitState *st = state + unit;
     uint32_t *ck = cand_key + (int64_t)unit * n_rows;
     uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
-    // the head of the candidate list is fetched before its length is known
-    uint32_t hk = 0, hi = 0;
-    if (tid < n_rows) {
-        hk = ck[tid];
-        hi = ci[tid];
+    // the head of the candidate list (what a list of ordinary length holds) is fetched before
+    // its length is known: one memory round trip less
+    constexpr int kHead = 4;
+    uint32_t hk[kHead], hi[kHead];
+#pragma unroll
+    for (int j = 0; j < kHead; ++j) {
+        const int i = tid + j * kFinalThreads;
+        hk[j] = hi[j] = 0;
+        if (i < n_rows) {
+            hk[j] = ck[i];
+            hi[j] = ci[i];
+        }
     }
     uint32_t n_c = st->cand_cnt;
     const uint32_t c_less = st->c_less;
@@ -822,18 +829,20 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     const uint32_t kk = (uint32_t)k_eff;
     uint32_t *io = idx_out + (int64_t)unit * idx_stride;
     uint32_t *ko = sel_keys ? sel_keys + (int64_t)unit * k_eff : nullptr;
-    const uint32_t *fk = ck, *fi = ci;
-    if (n_c <= (uint32_t)kCandLds) {
-        if ((uint32_t)tid < n_c) {
-            lck[tid] = hk;
-            lci[tid] = hi;
+    const bool staged = n_c <= (uint32_t)kCandLds;
+    if (staged) {
+#pragma unroll
+        for (int j = 0; j < kHead; ++j) {
+            const uint32_t i = (uint32_t)(tid + j * kFinalThreads);
+            if (i < n_c) {
+                lck[i] = hk[j];
+                lci[i] = hi[j];
+            }
         }
-        for (uint32_t i = tid + kFinalThreads; i < n_c; i += kFinalThreads) {
+        for (uint32_t i = tid + kHead * kFinalThreads; i < n_c; i += kFinalThreads) {
             lck[i] = ck[i];
             lci[i] = ci[i];
         }
-        fk = lck;
-        fi = lci;
     }
     __syncthreads();  // every thread has read the counters
     if (reinit) {
@@ -857,7 +866,7 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
         // (key, id).  The packed pairs sit in lh, padded with a sentinel to a multiple
         // of 8; the reads in the loop are wave-uniform 16-byte broadcasts.
         unsigned long long *comp = reinterpret_cast<unsigned long long *>(lh);
-        const unsigned long long mine = ((unsigned long long)hk << 32) | hi;
+        const unsigned long long mine = ((unsigned long long)hk[0] << 32) | hi[0];
         comp[tid] = (uint32_t)tid < n_c ? mine : ~0ull;
         __syncthreads();
         if ((uint32_t)tid < n_c) {
@@ -872,14 +881,17 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
                 }
             }
             if (rank < need) {
-                io[c_less + rank] = hi;
-                if (ko) ko[c_less + rank] = hk;
+                io[c_less + rank] = hi[0];
+                if (ko) ko[c_less + rank] = hk[0];
             }
         }
         return;
     }
-    dc_finalize_unit(fk, fi, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc,
-                     ko ? ko + c_less : nullptr);
+    // Two calls, so that the staged list is read with LDS instructions: through a pointer chosen
+    // at run time every access would be a flat one, and waiting for a flat load also waits for
+    // the stores issued above.
+    if (staged) dc_finalize_unit(lck, lci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc, ko ? ko + c_less : nullptr);
+    else dc_finalize_unit(ck, ci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc, ko ? ko + c_less : nullptr);
 }
 
 }  // namespace
