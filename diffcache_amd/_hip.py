@@ -29,7 +29,7 @@ SYMBOLS = (
     "dc_version", "dc_last_error", "dc_group_mean_bf16", "dc_score_bf16",
     "dc_topk_workspace_bytes", "dc_topk_select", "dc_gather_rows_bf16",
     "dc_attn_workspace_bytes", "dc_gather_attn_bf16", "dc_gather_attn_static_bf16", "dc_append_kv_bf16",
-    "dc_step_advance", "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
+    "dc_step_advance", "dc_step_state_advance", "dc_step_state_rollover", "dc_ingest_kv_bf16", "dc_layer_workspace_bytes", "dc_decode_layer",
     "dc_decode_layer_status", "dc_set_wait_limit", "dc_decode_layer_route", "dc_last_route",
     "dc_decode_layer_errors", "dc_one_kernel_guard",
     "dc_pq_build_lut", "dc_pq_adc_scan", "dc_score_gathered_bf16", "dc_compose_idx",
@@ -63,6 +63,7 @@ class LayerArgs(C.Structure):
         ("sketch_row_stride", C.c_int64),
         ("n_recent_dev", C.c_void_p),
         ("one_kernel", C.c_int),
+        ("region_hi_dev", C.c_void_p),
     ]
 
 
@@ -88,6 +89,8 @@ def _load() -> C.CDLL:
                                            i64, i64, i64, i64, i64, i64, f, p]),
         "dc_append_kv_bf16": (i, [p, p, p, p, i, i, i, i64, p, i64, i64, i64, i64, p]),
         "dc_step_advance": (i, [p, i, i, p]),
+        "dc_step_state_advance": (i, [p, i, i, p]),
+        "dc_step_state_rollover": (i, [p, i, i, p]),
         "dc_ingest_kv_bf16": (i, [p, p, i, i, i, i, i64, i64, i64, i64, p]),
         "dc_layer_workspace_bytes": (sz, [i, i, i, i, i, i]),
         "dc_decode_layer": (i, [C.POINTER(LayerArgs), p]),
@@ -492,6 +495,20 @@ def step_advance(counter: torch.Tensor, delta: int = 1, limit: int = 2 ** 31 - 1
     _check(lib.dc_step_advance(_counter(counter), delta, limit, _stream()))
 
 
+def step_state_advance(state: torch.Tensor, delta: int = 1, limit: int = 2 ** 31 - 1) -> None:
+    """dc_step_state_advance on a 4-element int32 device tensor [n_recent, region_hi, append_pos, overflow]."""
+    if not state.is_cuda or state.dtype != torch.int32 or state.numel() < 4 or not state.is_contiguous():
+        raise DiffCacheError("the step state must be a contiguous int32 tensor of 4 elements in GPU memory")
+    _check(lib.dc_step_state_advance(state.data_ptr(), delta, limit, _stream()))
+
+
+def step_state_rollover(state: torch.Tensor, moved: int, keep: int) -> None:
+    """dc_step_state_rollover: region_hi += moved, n_recent = keep, append_pos follows."""
+    if not state.is_cuda or state.dtype != torch.int32 or state.numel() < 4 or not state.is_contiguous():
+        raise DiffCacheError("the step state must be a contiguous int32 tensor of 4 elements in GPU memory")
+    _check(lib.dc_step_state_rollover(state.data_ptr(), moved, keep, _stream()))
+
+
 def ingest_kv(store: torch.Tensor, src: torch.Tensor, dst_pos: int = 0) -> None:
     """src (b, seq, h, hd) bf16 -> store[b, h, dst_pos + s, :]."""
     sb, sh, sr = _store_strides(store)
@@ -515,7 +532,7 @@ def layer_workspace_bytes(n_units: int, n_region: int, budget: int, group: int, 
 def _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
                 new_k=None, new_v=None, lse=None, mode=MODE_REF_DIST, order=ORDER_ANY, scale=None,
                 select_state_ready=False, scan_events=None, sketch=None, n_recent_dev=None,
-                one_kernel=ONE_KERNEL_AUTO) -> "LayerArgs":
+                one_kernel=ONE_KERNEL_AUTO, region_hi_dev=None) -> "LayerArgs":
     """struct dc_layer_args from tensors (the arguments of decode_layer), with their checks."""
     sb, sh, sr = _store_strides(store_k)
     if _store_strides(store_v) != (sb, sh, sr):
@@ -559,6 +576,7 @@ def _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores
         a.sketch_batch_stride, a.sketch_head_stride, a.sketch_row_stride = c.stride(0), c.stride(1), c.stride(2)
     a.n_recent_dev = _counter(n_recent_dev)
     a.one_kernel = one_kernel
+    a.region_hi_dev = _counter(region_hi_dev)
     a._keep = (q, store_k, store_v, new_k, new_v, out, lse, scores, idx_out, workspace, sketch, n_recent_dev)
     return a
 
@@ -573,15 +591,18 @@ def decode_layer(q: torch.Tensor, store_k: torch.Tensor, store_v: torch.Tensor, 
                  scan_events: Optional[Tuple[torch.cuda.Event, torch.cuda.Event]] = None,
                  sketch: Optional["Sketch"] = None,
                  n_recent_dev: Optional[torch.Tensor] = None,
-                 one_kernel: int = ONE_KERNEL_AUTO) -> torch.Tensor:
+                 one_kernel: int = ONE_KERNEL_AUTO,
+                 region_hi_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """score -> select -> attend for one layer, enqueued on the current stream.
     ``n_recent_dev``: the suffix length as a device-side int32 (``n_recent`` = capacity).
     ``select_state_ready``: see dc_layer_args in the header (skips the init kernel).
     ``sketch``: scan the 8-bit sketch of the keys instead of the keys (same result).
-    ``one_kernel``: ONE_KERNEL_* policy for short contexts (see the header)."""
+    ``one_kernel``: ONE_KERNEL_* policy for short contexts (see the header).
+    ``region_hi_dev``: the end of the retrieval region as a device-side int32 (``recent_lo`` = its
+    largest value), for captured steps that outlive a rollover of the recent window."""
     a = _layer_args(q, store_k, store_v, n_sink, recent_lo, n_recent, budget, scores, idx_out, out, workspace,
                     new_k, new_v, lse, mode, order, scale, select_state_ready, scan_events, sketch, n_recent_dev,
-                    one_kernel)
+                    one_kernel, region_hi_dev)
     _check(lib.dc_decode_layer(C.byref(a), _stream()))
     return out
 

@@ -81,6 +81,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     DC_REQUIRE(!(a->sketch_codes && a->scores), "dc_decode_layer: the sketch path needs scores == NULL");
     DC_REQUIRE(a->recent_lo >= a->n_sink, "dc_decode_layer: recent_lo %lld < n_sink %d",
                (long long)a->recent_lo, a->n_sink);
+    DC_REQUIRE(!(a->region_hi_dev && a->scores), "dc_decode_layer: region_hi_dev needs scores == NULL");
     const int n_units = a->n_b * a->n_h;
     if (n_units == 0) return DC_OK;
     const int64_t region64 = a->recent_lo - a->n_sink;
@@ -108,7 +109,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     }
     g_last_route = k_eff <= 0 ? DC_ROUTE_ATTEND_ONLY
                               : (a->scores ? DC_ROUTE_DENSE : (a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM));
-    if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY &&
+    if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY && !a->region_hi_dev &&
         dc_small_supported(n_units, region, k_eff, a->group, a->hd)) {
         // short context: the whole layer in one kernel whose blocks are all resident (ids in no
         // particular order); reads the bf16 keys, with or without a sketch.  The state is set up
@@ -134,12 +135,12 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
     if (k_eff > 0 && !a->scores && a->sketch_codes) {
         // streaming select over the 8-bit sketch, exact rescoring of the kept rows
         DC_REQUIRE(a->sketch_scale && a->sketch_resid, "dc_decode_layer: sketch_scale / sketch_resid missing");
-        rc = dc_score_select_sketch_bf16(
+        rc = dc_sketch_select_impl(
             k_region, a->sketch_codes + (int64_t)a->n_sink * a->sketch_row_stride, a->sketch_scale,
             a->sketch_resid, a->q, a->idx_out, a->idx_unit_stride, a->n_b, a->n_h, region, a->hd,
             a->kv_batch_stride, a->kv_head_stride, a->kv_row_stride, a->sketch_batch_stride,
             a->sketch_head_stride, a->sketch_row_stride, a->group, a->budget, a->mode, a->order,
-            ready, w.topk, w.topk_bytes, a->ev_scan_begin, a->ev_scan_end, stream);
+            ready, w.topk, w.topk_bytes, a->ev_scan_begin, a->ev_scan_end, stream, a->region_hi_dev, a->n_sink);
         if (rc) return rc;
     } else if (k_eff > 0 && !a->scores) {
         // no dense scores wanted: streaming score + select
@@ -148,9 +149,9 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
             if (rc) return rc;
         }
         if (a->ev_scan_begin) (void)hipEventRecord((hipEvent_t)a->ev_scan_begin, st);
-        rc = dc_score_prune_bf16(k_region, a->q, a->n_b, a->n_h, region, a->hd, a->kv_batch_stride,
-                                 a->kv_head_stride, a->kv_row_stride, a->group, a->budget, a->mode, w.topk,
-                                 w.topk_bytes, stream);
+        rc = dc_score_prune_launch(k_region, a->q, a->n_b, a->n_h, region, a->hd, a->kv_batch_stride,
+                                   a->kv_head_stride, a->kv_row_stride, a->group, a->budget, a->mode, w.topk,
+                                   w.topk_bytes, stream, a->region_hi_dev, a->n_sink);
         if (rc) return rc;
         if (a->ev_scan_end) (void)hipEventRecord((hipEvent_t)a->ev_scan_end, st);
         rc = dc_sparse_select(a->idx_out, a->idx_unit_stride, n_units, region, a->budget, a->mode, a->order,
@@ -171,11 +172,11 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
                             region, a->budget, a->mode, a->order, w.hist, w.topk, w.topk_bytes, stream);
         if (rc) return rc;
     }
-    rc = dc_gather_attn_bf16(a->q, a->k, a->v, a->idx_out, a->new_k, a->new_v, a->out, a->lse, a->n_b,
-                             a->n_h, a->group, a->hd, k_eff, a->idx_unit_stride, nullptr, a->n_sink, a->n_sink,
-                             a->recent_lo, a->n_recent, a->n_recent_dev, a->kv_batch_stride, a->kv_head_stride,
-                             a->kv_row_stride, a->kv_batch_stride, a->kv_head_stride,
-                             a->kv_row_stride, a->scale, w.attn, w.attn_bytes, stream);
+    rc = dc_gather_attn_common("dc_decode_layer", a->q, a->k, a->v, a->idx_out, a->new_k, a->new_v, a->out, a->lse,
+                               a->n_b, a->n_h, a->group, a->hd, k_eff, a->idx_unit_stride, nullptr, a->n_sink,
+                               a->n_sink, a->recent_lo, a->n_recent, a->n_recent_dev, a->kv_batch_stride,
+                               a->kv_head_stride, a->kv_row_stride, a->kv_batch_stride, a->kv_head_stride,
+                               a->kv_row_stride, a->scale, w.attn, w.attn_bytes, stream, a->region_hi_dev);
     return rc;
 }
 
@@ -188,7 +189,7 @@ extern "C" int dc_decode_layer_route(const dc_layer_args *a) {
     const int k_eff = a->budget < region ? a->budget : region;
     if (n_units == 0 || k_eff <= 0) return DC_ROUTE_ATTEND_ONLY;
     if (a->scores) return DC_ROUTE_DENSE;
-    if (a->order == DC_ORDER_ANY && a->one_kernel != DC_ONE_KERNEL_NEVER &&
+    if (a->order == DC_ORDER_ANY && a->one_kernel != DC_ONE_KERNEL_NEVER && !a->region_hi_dev &&
         dc_small_supported(n_units, region, k_eff, a->group, a->hd))
         return DC_ROUTE_ONE_KERNEL;
     return a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;

@@ -165,17 +165,17 @@ extern "C" size_t dc_attn_workspace_bytes(int n_units, int group, int hd, int n_
     return a > b ? a : b;
 }
 
-namespace {
-
-// Argument checks and the two launches shared by dc_gather_attn_bf16 (caller's workspace) and
-// dc_gather_attn_static_bf16 (the library's static scratch array).
-int gather_attn_common(const char *who, const void *q, const void *k, const void *v, const uint32_t *idx,
+// Argument checks and the two launches shared by dc_gather_attn_bf16 (caller's workspace),
+// dc_gather_attn_static_bf16 (the library's static scratch array) and dc_decode_layer.
+// recent_lo_dev: null, or a device word holding the first row of the suffix at the time the
+// kernels run (recent_lo is then its largest value).
+int dc_gather_attn_common(const char *who, const void *q, const void *k, const void *v, const uint32_t *idx,
                        const void *new_k, const void *new_v, void *out, float *lse, int n_b, int n_h,
                        int group, int hd, int n_idx, int64_t idx_unit_stride, const uint32_t *n_idx_unit,
                        int64_t region_lo, int n_sink, int64_t recent_lo, int n_recent,
                        const int32_t *n_recent_dev, int64_t ksb, int64_t ksh, int64_t ksr, int64_t vsb,
                        int64_t vsh, int64_t vsr, float scale, void *workspace, size_t workspace_bytes,
-                       void *stream) {
+                       void *stream, const int32_t *recent_lo_dev) {
     DC_REQUIRE(q && k && v && out, "%s: null pointer", who);
     DC_REQUIRE(n_b >= 0 && n_h >= 1 && n_idx >= 0 && n_sink >= 0 && n_recent >= 0,
                "%s: bad sizes", who);
@@ -220,6 +220,7 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     aa.ws_ml = w.ml;
     aa.n_idx_unit = n_idx_unit;
     aa.n_recent_dev = n_recent_dev;
+    aa.recent_lo_dev = recent_lo_dev;
     aa.n_h = n_h;
     aa.n_idx = n_idx;
     aa.idx_stride = idx_unit_stride;
@@ -249,6 +250,8 @@ int gather_attn_common(const char *who, const void *q, const void *k, const void
     return DC_OK;
 }
 
+namespace {
+
 // Scratch of the allocation-free entry point: the per-split (m, l, acc) partials.  One copy
 // per GPU, held until the process ends.  In host code the array's name is only a handle for
 // hipGetSymbolAddress; the device address is looked up once per device and kept.
@@ -270,10 +273,10 @@ extern "C" int dc_gather_attn_bf16(const void *q, const void *k, const void *v, 
                                    int64_t ksb, int64_t ksh,
                                    int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
                                    void *workspace, size_t workspace_bytes, void *stream) {
-    return gather_attn_common("dc_gather_attn_bf16", q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group,
-                              hd, n_idx, idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo,
-                              n_recent, n_recent_dev, ksb, ksh, ksr, vsb, vsh, vsr, scale, workspace, workspace_bytes,
-                              stream);
+    return dc_gather_attn_common("dc_gather_attn_bf16", q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group,
+                                 hd, n_idx, idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo,
+                                 n_recent, n_recent_dev, ksb, ksh, ksr, vsb, vsh, vsr, scale, workspace, workspace_bytes,
+                                 stream, nullptr);
 }
 
 extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const void *v, const uint32_t *idx,
@@ -320,9 +323,9 @@ extern "C" int dc_gather_attn_static_bf16(const void *q, const void *k, const vo
     }
     // Every split slot the merge reads is written by the attention kernel of the same call, so
     // nothing has to start at zero; the contents of the previous call are simply overwritten.
-    return gather_attn_common(who, q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group, hd, n_idx,
-                              idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo, n_recent, n_recent_dev,
-                              ksb, ksh, ksr, vsb, vsh, vsr, scale, ptr, kStaticScratchBytes, stream);
+    return dc_gather_attn_common(who, q, k, v, idx, new_k, new_v, out, lse, n_b, n_h, group, hd, n_idx,
+                                 idx_unit_stride, n_idx_unit, region_lo, n_sink, recent_lo, n_recent, n_recent_dev,
+                                 ksb, ksh, ksr, vsb, vsh, vsr, scale, ptr, kStaticScratchBytes, stream, nullptr);
 }
 
 extern "C" int dc_gather_rows_bf16(const void *k, const void *v, const uint32_t *idx, void *out_k,

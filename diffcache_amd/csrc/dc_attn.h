@@ -76,6 +76,7 @@ struct AttnArgs {
     float *ws_acc, *ws_ml;
     const uint32_t *n_idx_unit;
     const int32_t *n_recent_dev;
+    const int32_t *recent_lo_dev;  // null, or the first row of the suffix as a device word (recent_lo: its largest value)
     int n_h, n_idx;
     int64_t idx_stride, region_lo;
     int n_sink;
@@ -110,6 +111,7 @@ __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int s
     const int r0 = split * ROWS;
     const int n_idx = a.n_idx, n_sink = a.n_sink;
     int n_recent = a.n_recent, n_total = a.n_total;
+    const int64_t recent_lo = a.recent_lo_dev ? (int64_t)*a.recent_lo_dev : a.recent_lo;
 
     // The length of the recent window may live on the device (the role of cache_seqlens in
     // base.py:134-142): n_recent is then its capacity, which sized the grid, and the rows
@@ -143,7 +145,7 @@ __device__ __forceinline__ void dc_attn_split(const AttnArgs &a, int unit, int s
             } else if (vj < n_idx + n_sink) {
                 r = (uint32_t)(vj - n_idx);
             } else if (vj < n_idx + n_sink + n_recent) {
-                r = (uint32_t)(a.recent_lo + (vj - n_idx - n_sink));
+                r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
             } else {
                 r = kNewToken;
             }
@@ -342,6 +344,7 @@ __device__ __forceinline__ void dc_attn_split_mfma(const AttnArgs &a, int G, int
     const int q = lane >> 4, c = lane & 15;
     const int n_idx = a.n_idx, n_sink = a.n_sink;
     int n_recent = a.n_recent, n_total = a.n_total;
+    const int64_t recent_lo = a.recent_lo_dev ? (int64_t)*a.recent_lo_dev : a.recent_lo;
     if (a.n_recent_dev) {  // the window's length may live on the device (cache_seqlens, base.py:134-142)
         int cur = *a.n_recent_dev;
         cur = cur < 0 ? 0 : (cur < n_recent ? cur : n_recent);
@@ -365,7 +368,7 @@ __device__ __forceinline__ void dc_attn_split_mfma(const AttnArgs &a, int G, int
         if (live(vj)) {
             if (vj < n_idx) r = (uint32_t)(a.region_lo + a.idx[(int64_t)unit * a.idx_stride + vj]);
             else if (vj < n_idx + n_sink) r = (uint32_t)(vj - n_idx);
-            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(a.recent_lo + (vj - n_idx - n_sink));
+            else if (vj < n_idx + n_sink + n_recent) r = (uint32_t)(recent_lo + (vj - n_idx - n_sink));
             else r = kNewToken;
         }
         rowk[t] = r;

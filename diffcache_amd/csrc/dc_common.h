@@ -39,7 +39,25 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
                           const float *resid, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb,
                           int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group, int budget,
                           int mode, int state_ready, void *workspace, size_t workspace_bytes,
-                          void *ev_scan_begin, void *ev_scan_end, void *stream);
+                          void *ev_scan_begin, void *ev_scan_end, void *stream, const int32_t *hi_dev = nullptr,
+                          int lo_row = 0);
+// fused.hip: the bf16 scan of the streaming route (dc_score_prune_bf16 with an optional device-side region end)
+int dc_score_prune_launch(const void *k, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb, int64_t sh,
+                          int64_t sr, int q_group, int budget, int mode, void *workspace, size_t workspace_bytes,
+                          void *stream, const int32_t *hi_dev, int lo_row);
+// fused.hip: dc_score_select_sketch_bf16 with an optional device-side region end
+int dc_sketch_select_impl(const void *k, const uint8_t *codes, const float *scale, const float *resid, const void *q,
+                          uint32_t *idx_out, int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                          int64_t sb, int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group,
+                          int budget, int mode, int order, int state_ready, void *workspace, size_t workspace_bytes,
+                          void *ev_scan_begin, void *ev_scan_end, void *stream, const int32_t *hi_dev, int lo_row);
+// attn.hip: dc_gather_attn_bf16 with an optional device-side start of the suffix
+int dc_gather_attn_common(const char *who, const void *q, const void *k, const void *v, const uint32_t *idx,
+                          const void *new_k, const void *new_v, void *out, float *lse, int n_b, int n_h, int group,
+                          int hd, int n_idx, int64_t idx_unit_stride, const uint32_t *n_idx_unit, int64_t region_lo,
+                          int n_sink, int64_t recent_lo, int n_recent, const int32_t *n_recent_dev, int64_t ksb,
+                          int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
+                          void *workspace, size_t workspace_bytes, void *stream, const int32_t *recent_lo_dev);
 // small.hip: a whole decode layer in one kernel, for short contexts
 bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd);
 size_t dc_small_workspace_bytes(int n_units, int region, int group, int hd);
@@ -164,6 +182,15 @@ __device__ __forceinline__ float dc_group_sum(float v) {
     v = dc_row16_sum(v);
     if (LPR == 32) v += __shfl_xor(v, 16, 64);
     return v;
+}
+
+// Rows of a retrieval region that are live.  The kernels' grids and lists are laid out for
+// n_cap rows; with hi_dev the region ends at the row that device word names (it moves up when the
+// recent window is rolled over, between replays of a captured step), lo_row being its first row.
+__device__ __forceinline__ int dc_live_rows(int n_cap, const int32_t *hi_dev, int lo_row) {
+    if (!hi_dev) return n_cap;
+    const int v = *hi_dev - lo_row;
+    return v < 0 ? 0 : (v < n_cap ? v : n_cap);
 }
 
 // 8 bf16 (one 16-byte load) dotted with 8 fp32 query values, added to acc

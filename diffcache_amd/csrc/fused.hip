@@ -134,9 +134,9 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
 template <int HD>
 __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     const uint16_t *__restrict__ K, const uint16_t *__restrict__ Q, uint32_t *__restrict__ hist,
-    UnitState *__restrict__ state, uint2 *__restrict__ surv, int n_units, int n_h, int n_rows,
+    UnitState *__restrict__ state, uint2 *__restrict__ surv, int n_units, int n_h, int n_cap,
     int64_t sb, int64_t sh, int64_t sr, int q_group, int mode, int k_eff, int small_chunks,
-    int big_steps) {
+    int big_steps, const int32_t *__restrict__ hi_dev, int lo_row) {
     constexpr int LPR = HD / 8;
     constexpr int CH = LPR < 16 ? LPR : 16;
     __shared__ uint32_t lhist[DC_HIST_BINS];
@@ -144,6 +144,7 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     __shared__ uint32_t wtot[kThreads / 64 + 1];
     __shared__ uint32_t s_wcnt[kThreads / 64];
     __shared__ uint32_t s_base;
+    const int n_rows = dc_live_rows(n_cap, hi_dev, lo_row);
 
     const int unit = blockIdx.x % n_units;
     const int chunk = blockIdx.x / n_units;
@@ -162,6 +163,7 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
               : (int64_t)small_chunks * kRowsPerBlockStep + (int64_t)big_id * big_steps * kRowsPerBlockStep;
     const int steps = small ? 1 : big_steps;
 
+    if (block_row0 >= n_rows) return;  // the grid is laid out for n_cap rows
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
 
     const uint16_t *Ku = K + b * sb + h * sh + col * 8;
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(kThreads) void score_prune_kernel(
     // every 4th small block and every 8th large one refresh the running threshold
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
-                       surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
+                       surv + (int64_t)unit * n_cap, refresh, (uint32_t)k_eff);
 }
 
 // sum over aligned groups of LPR lanes (4, 8 or 16)
@@ -263,9 +265,11 @@ template <int HD, bool SHARED_POLL>
 __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kernel(
     const uint8_t *__restrict__ C, const uint16_t *__restrict__ Q, const float *__restrict__ scale,
     const float *__restrict__ resid, uint32_t *__restrict__ hist, UnitState *__restrict__ state,
-    uint2 *__restrict__ surv, int n_units, int n_h, int n_rows, int64_t cb, int64_t ch, int64_t cr,
-    int q_group, int mode, int k_eff, int small_chunks, int big_steps) {
+    uint2 *__restrict__ surv, int n_units, int n_h, int n_cap, int64_t cb, int64_t ch, int64_t cr,
+    int q_group, int mode, int k_eff, int small_chunks, int big_steps, const int32_t *__restrict__ hi_dev,
+    int lo_row) {
     constexpr int LPR = HD / 16;  // lanes per row, 16 code bytes each
+    const int n_rows = dc_live_rows(n_cap, hi_dev, lo_row);
     __shared__ uint32_t lhist[DC_HIST_BINS];
     __shared__ uint2 stage[kStage];
     __shared__ uint32_t s_tb;  // the block's copy of the unit's running threshold bucket
@@ -288,6 +292,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
               : (int64_t)small_chunks * kRowsPerBlockStep + (int64_t)big_id * big_steps * kRowsPerBlockStep;
     const int steps = small ? 1 : big_steps;
 
+    if (block_row0 >= n_rows) return;  // the grid is laid out for n_cap rows
     for (int i = tid; i < DC_HIST_BINS; i += kThreads) lhist[i] = 0;
 
     const uint8_t *Cu = C + b * cb + h * ch + col * 16;
@@ -441,7 +446,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     }
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
     prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
-                       surv + (int64_t)unit * n_rows, refresh, (uint32_t)k_eff);
+                       surv + (int64_t)unit * n_cap, refresh, (uint32_t)k_eff);
 }
 
 // The same scan for the PQ baseline: a key's score is its ADC score (dc_pq.h), read
@@ -966,6 +971,16 @@ extern "C" int dc_select_state_init(int n_units, int n_rows, int budget, void *w
 extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_h, int n_rows, int hd,
                                    int64_t sb, int64_t sh, int64_t sr, int q_group, int budget,
                                    int mode, void *workspace, size_t workspace_bytes, void *stream) {
+    return dc_score_prune_launch(k, q, n_b, n_h, n_rows, hd, sb, sh, sr, q_group, budget, mode, workspace,
+                                 workspace_bytes, stream, nullptr, 0);
+}
+
+// hi_dev: null, or a device word holding the row at which the region ends at the time the kernel
+// runs (lo_row: its first row); n_rows is then the capacity that the grid and the lists are laid
+// out for.
+int dc_score_prune_launch(const void *k, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb, int64_t sh,
+                          int64_t sr, int q_group, int budget, int mode, void *workspace, size_t workspace_bytes,
+                          void *stream, const int32_t *hi_dev, int lo_row) {
     DC_REQUIRE(k && q, "dc_score_prune_bf16: null pointer");
     DC_REQUIRE(q_group >= 1, "dc_score_prune_bf16: bad q_group");
     DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "dc_score_prune_bf16: head_dim %d not in {64,128,256}", hd);
@@ -985,7 +1000,7 @@ extern "C" int dc_score_prune_bf16(const void *k, const void *q, int n_b, int n_
     hipLaunchKernelGGL(score_prune_kernel<HD>, dim3((unsigned)p.blocks), dim3(kThreads), 0, st,    \
                        (const uint16_t *)k, (const uint16_t *)q, w.hist, w.state, w.surv,          \
                        p.n_units, n_h, n_rows, sb, sh, sr, q_group, mode, p.k_eff, p.small_chunks,  \
-                       p.big_steps)
+                       p.big_steps, hi_dev, lo_row)
     if (hd == 64) DC_LAUNCH_SP(64);
     else if (hd == 128) DC_LAUNCH_SP(128);
     else DC_LAUNCH_SP(256);
@@ -1072,7 +1087,7 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
                           const float *resid, const void *q, int n_b, int n_h, int n_rows, int hd, int64_t sb,
                           int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group, int budget,
                           int mode, int state_ready, void *workspace, size_t workspace_bytes,
-                          void *ev_scan_begin, void *ev_scan_end, void *stream) {
+                          void *ev_scan_begin, void *ev_scan_end, void *stream, const int32_t *hi_dev, int lo_row) {
     DC_REQUIRE(k && codes && scale && resid && q, "%s: null pointer", who);
     DC_REQUIRE(q_group >= 1, "%s: bad q_group", who);
     DC_REQUIRE(hd == 64 || hd == 128 || hd == 256, "%s: head_dim %d not in {64,128,256}", who, hd);
@@ -1103,7 +1118,7 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
 #define DC_LAUNCH_SK(HD, SP)                                                                        \
     hipLaunchKernelGGL((sketch_prune_kernel<HD, SP>), dim3((unsigned)p.blocks), dim3(kThreads), 0, st,  \
                        codes, (const uint16_t *)q, scale, resid, w.hist, w.state, w.surv, p.n_units,    \
-                       n_h, n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps)
+                       n_h, n_rows, cb, ch, cr, q_group, mode, p.k_eff, p.small_chunks, p.big_steps, hi_dev, lo_row)
     const bool shared_poll = p.n_units <= kSharedPollUnits;
     if (hd == 64 && shared_poll) DC_LAUNCH_SK(64, true);
     else if (hd == 64) DC_LAUNCH_SK(64, false);
@@ -1124,12 +1139,24 @@ extern "C" int dc_score_select_sketch_bf16(const void *k, const uint8_t *codes, 
                                            int64_t cr, int q_group, int budget, int mode, int order,
                                            int state_ready, void *workspace, size_t workspace_bytes,
                                            void *ev_scan_begin, void *ev_scan_end, void *stream) {
+    return dc_sketch_select_impl(k, codes, scale, resid, q, idx_out, idx_unit_stride, n_b, n_h, n_rows, hd, sb, sh, sr,
+                                 cb, ch, cr, q_group, budget, mode, order, state_ready, workspace, workspace_bytes,
+                                 ev_scan_begin, ev_scan_end, stream, nullptr, 0);
+}
+
+// hi_dev, lo_row: as in dc_score_prune_launch.  Only the scan needs the live length: the passes
+// after it work on the lists the scan left, whose capacity is n_rows.
+int dc_sketch_select_impl(const void *k, const uint8_t *codes, const float *scale, const float *resid, const void *q,
+                          uint32_t *idx_out, int64_t idx_unit_stride, int n_b, int n_h, int n_rows, int hd,
+                          int64_t sb, int64_t sh, int64_t sr, int64_t cb, int64_t ch, int64_t cr, int q_group,
+                          int budget, int mode, int order, int state_ready, void *workspace, size_t workspace_bytes,
+                          void *ev_scan_begin, void *ev_scan_end, void *stream, const int32_t *hi_dev, int lo_row) {
     const char *who = "dc_score_select_sketch_bf16";
     DC_REQUIRE(idx_out, "%s: null pointer", who);
     DC_REQUIRE(order >= DC_ORDER_ANY && order <= DC_ORDER_INDEX, "%s: bad order %d", who, order);
     int rc = dc_sketch_scan_launch(who, k, codes, scale, resid, q, n_b, n_h, n_rows, hd, sb, sh, sr, cb, ch, cr,
                                    q_group, budget, mode, state_ready, workspace, workspace_bytes,
-                                   ev_scan_begin, ev_scan_end, stream);
+                                   ev_scan_begin, ev_scan_end, stream, hi_dev, lo_row);
     if (rc) return rc;
     FusedPlan p;
     rc = plan_fused(who, n_b, n_h, n_rows, budget, &p);

@@ -35,6 +35,27 @@ __global__ void step_advance_kernel(int32_t *counter, int delta, int limit) {
     }
 }
 
+// The step state of a sequence as four device words (dc_step_state in the header): one thread.
+__global__ void step_state_advance_kernel(int32_t *s, int delta, int limit) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        int64_t n = (int64_t)s[0] + delta;
+        if (n > limit) {  // the window is full: this token has no row (the caller had to roll it over)
+            s[3] = 1;
+            n = limit;
+        }
+        if (n < 0) n = 0;
+        s[0] = (int32_t)n;
+        s[2] = s[1] + (int32_t)n;
+    }
+}
+__global__ void step_state_rollover_kernel(int32_t *s, int moved, int keep) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        s[1] += moved;
+        s[0] = keep;
+        s[2] = s[1] + keep;
+    }
+}
+
 // src (n_b, seq, n_h, hd) -> store[b, h, dst_pos + s, :]; one 16-byte chunk per
 // thread, threads ordered like the source so reads are fully coalesced and
 // writes land as whole rows
@@ -81,6 +102,22 @@ extern "C" int dc_step_advance(int32_t *counter, int delta, int limit, void *str
     DC_REQUIRE(limit >= 0, "dc_step_advance: negative limit");
     hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, counter, delta, limit);
     DC_CHECK_LAUNCH("dc_step_advance");
+    return DC_OK;
+}
+
+extern "C" int dc_step_state_advance(int32_t *state, int delta, int limit, void *stream) {
+    DC_REQUIRE(state, "dc_step_state_advance: null pointer");
+    DC_REQUIRE(limit >= 0, "dc_step_state_advance: negative limit");
+    hipLaunchKernelGGL(step_state_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, state, delta, limit);
+    DC_CHECK_LAUNCH("dc_step_state_advance");
+    return DC_OK;
+}
+
+extern "C" int dc_step_state_rollover(int32_t *state, int moved, int keep, void *stream) {
+    DC_REQUIRE(state, "dc_step_state_rollover: null pointer");
+    DC_REQUIRE(moved >= 0 && keep >= 0, "dc_step_state_rollover: negative count");
+    hipLaunchKernelGGL(step_state_rollover_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, state, moved, keep);
+    DC_CHECK_LAUNCH("dc_step_state_rollover");
     return DC_OK;
 }
 

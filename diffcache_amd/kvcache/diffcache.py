@@ -25,11 +25,13 @@ own attention over ``get_kvcache()``.
 reference: score -> select -> attention straight from the store (one C call),
 replacing the ``flash_attn_with_kvcache`` call of ``base.py:134-142`` as well.
 
-Step state.  The length of the recent window lives in a one-element int32 tensor on the
-device (``step_state``), like the ``cache_seqlens`` tensor the reference hands to
-flash-attn (``base.py:134-142,150-152``): ``decode_attention`` appends at, and attends up
-to, the row that counter names, and advances it after the last layer.  A call captured
-in a HIP graph therefore stays right on every replay; after replays the host's mirror
+Step state.  The length of the recent window, the row at which the retrieval region ends
+and the row the next token is appended at live in a small int32 tensor on the device
+(``dc_step_state`` of the header; ``step_state`` is the view of its first word), like the
+``cache_seqlens`` tensor the reference hands to flash-attn (``base.py:134-142,150-152``):
+a captured ``decode_attention`` appends at, scans up to and attends over the rows those
+words name, and advances them after the last layer.  A call captured in a HIP graph
+therefore stays right on every replay; after replays the host's mirror
 (``kvbuf_suffix_len``) is brought up to date with ``advance_host_step``.
 
 Rollover.  The reference never moves tokens out of the recent window into its index
@@ -37,10 +39,13 @@ Rollover.  The reference never moves tokens out of the recent window into its in
 sequence ends after ``kvbuf_suffix_maxlen - kvbuf_suffix_len`` tokens.  Here the rows are
 already in the store, so when the window is full the region boundary simply moves: the
 oldest rows of the window join the retrieval region (their sketch rows are added with the
-fitted scales kept) and the window shrinks back to its initial length.  This is a
-host-side event between two decode steps (``rollover``; ``generation`` counts them):
-graphs captured before it must be captured again, since the region length is a launch
-parameter.
+fitted scales kept) and the window shrinks back to its initial length (``rollover``;
+``generation`` counts them).  The call only enqueues work on the stream -- sketch rows, two
+device words -- so it may sit between two replays of a captured step, and a step that was
+captured while the region held at least ``retrieval_budget`` rows stays valid across it,
+as the reference's graphs do for a whole generation (``base.py:46-55``); one captured with
+a shorter region, or with ``use_k_check``, has the region's end as a launch parameter and
+must be captured again (``captured_region_on_device`` tells which).
 
 Two options beyond the reference's arguments.  ``key_sketch`` (default on): an
 8-bit sketch of the keys is built at prefill and the scans read it instead of
@@ -172,8 +177,11 @@ class DiffCache:
         self._attn_ws: Optional[torch.Tensor] = None
         self._prefix0 = kvbuf_prefix_len
         self._suffix0 = kvbuf_suffix_len
-        # device-side length of the recent window (the host mirror is kvbuf_suffix_len)
-        self.step_state = torch.full((1,), kvbuf_suffix_len, device=self.device, dtype=torch.int32)
+        # device-side step state [n_recent, region_hi, append_pos, overflow] (dc_step_state); the
+        # host mirrors are kvbuf_suffix_len and _region()
+        self._state = torch.zeros((4,), device=self.device, dtype=torch.int32)
+        self.step_state = self._state[0:1]
+        self.captured_region_on_device: Optional[bool] = None   # of the last captured decode_attention
         # suffix rows that are present in kstore / vstore: all of them on the native route,
         # only the prompt's on the hook route (the harness's attention call writes the new
         # tokens into kbuf / vbuf, as flash_attn_with_kvcache does for the reference)
@@ -204,8 +212,22 @@ class DiffCache:
         return self._ws
 
     def _set_suffix_len(self, n: int) -> None:
+        """Window length and, from the host's view of the region, the whole device-side state."""
         self.kvbuf_suffix_len = n
-        self.step_state.fill_(n)
+        _, hi = self._region()
+        self._state[0:1].fill_(n)
+        self._state[1:2].fill_(hi)
+        self._state[2:3].fill_(hi + n)
+
+    def check_status(self) -> None:
+        """Waits for the device and raises if a decoded token was dropped because the recent
+        window was full when its step ran (replays of a captured step beyond the window's
+        capacity without ``rollover()``), or if a one-kernel launch gave up a wait."""
+        n_recent, region_hi, append_pos, overflow = self._state.tolist()
+        hip.require(overflow == 0, "a decode step ran with a full recent window: its token was not stored "
+                                   "(call rollover() before the step that finds the window full)")
+        self._note_failures()
+        hip.require(self.failed_steps == 0, f"{self.failed_steps} one-kernel launches gave up a wait; their outputs were NaN")
 
     def advance_host_step(self, steps: int = 1) -> None:
         """After ``steps`` replays of a captured decode step: bring the host's mirror of the
@@ -220,8 +242,9 @@ class DiffCache:
 
     def rollover(self) -> int:
         """Move the oldest rows of the recent window into the retrieval region (see the module
-        docstring).  Host-side, between two decode steps, never under graph capture.  Returns
-        the number of rows moved."""
+        docstring).  Between two decode steps (or two replays of a captured one), never under
+        graph capture; only enqueues work on the current stream.  Returns the number of rows
+        moved."""
         hip.require(not torch.cuda.is_current_stream_capturing(), "rollover() cannot be captured in a graph")
         keep = min(self._suffix0, self.kvbuf_suffix_maxlen - 1)
         moved = self.kvbuf_suffix_len - keep
@@ -243,7 +266,8 @@ class DiffCache:
             self.kbuf[l][:, :, b0 + p:b0 + p + keep].copy_(ks[:, :, hi + moved:hi + s])
             self.vbuf[l][:, :, b0 + p:b0 + p + keep].copy_(vs[:, :, hi + moved:hi + s])
         self.retrieval_region_len += moved
-        self._set_suffix_len(keep)
+        self.kvbuf_suffix_len = keep
+        hip.step_state_rollover(self._state, moved, keep)      # the device's view, in stream order
         self._store_suffix_rows = keep
         self._ws_ready = False
         self._hook_ws_ready = False
@@ -271,9 +295,9 @@ class DiffCache:
         prefix_len = min(self._prefix0, seq_len)                    # diffcache.py:163
         suffix_len = min(self._suffix0, seq_len - prefix_len)       # diffcache.py:169
         self.kvbuf_prefix_len = prefix_len
+        self.retrieval_region_len = seq_len - prefix_len - suffix_len
         self._set_suffix_len(suffix_len)
         self._store_suffix_rows = suffix_len
-        self.retrieval_region_len = seq_len - prefix_len - suffix_len
         if self.key_sketch and self.retrieval_region_len > 0:
             self.sketch[layer_idx].build(self.kstore[layer_idx], prefix_len, self.retrieval_region_len)
 
@@ -336,7 +360,7 @@ class DiffCache:
                     "the recent window is full (kvbuf_suffix_maxlen)")       # diffcache.py:221
         if layer_idx == self.num_layers - 1:
             self.kvbuf_suffix_len += 1                                       # diffcache.py:222-223
-            hip.step_advance(self.step_state, 1, self.kvbuf_suffix_maxlen)
+            hip.step_state_advance(self._state, 1, self.kvbuf_suffix_maxlen)
 
     def decode_post_query_operation(self, layer_idx: int) -> None:
         """Selected rows into kbuf/vbuf[:, :, budget - len : budget] (diffcache.py:196-209)."""
@@ -377,9 +401,21 @@ class DiffCache:
             nk = nk.contiguous()
         if not nv.is_contiguous():
             nv = nv.contiguous()
-        # the token's row: hi + (device-side window length); never past the window's capacity
-        hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], nk, nv, hi, pos_dev=self.step_state,
-                      pos_end=min(hi + self.kvbuf_suffix_maxlen, self.max_length))
+        # Under capture the region's end is read from the device wherever the path allows it (a
+        # region of at least `budget` rows, no k-check), so that the graph outlives a rollover:
+        # launches and workspace are then laid out for the longest region the store can hold.
+        dev_region = capturing and not self.use_k_check and hi - lo >= self.retrieval_budget > 0
+        if capturing:
+            self.captured_region_on_device = dev_region
+        hi_cap = self.max_length - self.kvbuf_suffix_maxlen
+        if dev_region:
+            # the token's row is the device's append position; never past the end of the store
+            hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], nk, nv, 0, pos_dev=self._state[2:3],
+                          pos_end=self.max_length)
+        else:
+            # the token's row: hi + (device-side window length); never past the window's capacity
+            hip.append_kv(self.kstore[layer_idx], self.vstore[layer_idx], nk, nv, hi, pos_dev=self.step_state,
+                          pos_end=min(hi + self.kvbuf_suffix_maxlen, self.max_length))
         if out is None:
             if self._attn_out is None:
                 self._attn_out = torch.empty((b, hq, hd), device=self.device, dtype=torch.bfloat16)
@@ -389,17 +425,21 @@ class DiffCache:
             self._decode_attention_k_check(layer_idx, q, nk, nv, out, ws)
         else:
             # attended: [selected | prefix | the window's rows before this token | this token]
-            hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi,
+            # (a call with the region's end on the device has other launch sizes than one without:
+            #  neither leaves the select state ready for the other)
+            tag = (order, dev_region)
+            hip.decode_layer(q, self.kstore[layer_idx], self.vstore[layer_idx], lo, hi_cap if dev_region else hi,
                              self.kvbuf_suffix_maxlen, self.retrieval_budget, None, self.idx[layer_idx], out, ws,
                              nk, nv, mode=self.mode, order=order,
-                             select_state_ready=self._ws_ready and self._ws_order == order,
+                             select_state_ready=self._ws_ready and self._ws_order == tag,
                              sketch=self.sketch[layer_idx], n_recent_dev=self.step_state,
-                             one_kernel=self.one_kernel)
+                             one_kernel=self.one_kernel,
+                             region_hi_dev=self._state[1:2] if dev_region else None)
             self._ws_ready = True
-            self._ws_order = order      # the state is left ready for a call of the same order only
+            self._ws_order = tag        # the state is left ready for a call of the same kind only
             self._hook_ws_ready = False
         if layer_idx == self.num_layers - 1:
-            hip.step_advance(self.step_state, 1, self.kvbuf_suffix_maxlen)
+            hip.step_state_advance(self._state, 1, self.kvbuf_suffix_maxlen)
             if not capturing:       # a captured step is counted when it is replayed (advance_host_step)
                 self.kvbuf_suffix_len += 1
                 self._store_suffix_rows += 1
@@ -493,9 +533,9 @@ class DiffCache:
             metadata = json.load(f)
         self.r_sq = metadata["r_sq"]
         self.kvbuf_prefix_len = metadata["kvbuf_prefix_len"]
+        self.retrieval_region_len = metadata["retrieval_region_len"]
         self._set_suffix_len(metadata["kvbuf_suffix_len"])
         self._store_suffix_rows = self.kvbuf_suffix_len
-        self.retrieval_region_len = metadata["retrieval_region_len"]
         b0, p, s = self.retrieval_budget, self.kvbuf_prefix_len, self.kvbuf_suffix_len
         lo, hi = self._region()
         for layer_idx in range(self.num_layers):

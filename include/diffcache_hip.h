@@ -288,6 +288,29 @@ int dc_append_kv_bf16(void *k_store, void *v_store, const void *new_k, const voi
 int dc_step_advance(int32_t *counter, int delta, int limit, void *stream);
 
 /*
+ * The whole per-sequence step state as four device words, for a decode step that is captured
+ * once and replayed for the whole generation (the reference captures its per-layer graphs once,
+ * src/diffcache/base.py:46-55,116-148, and its data layer takes every decoded token as it comes,
+ * diffcache_cpu/src/lib.rs:352-369):
+ *   n_recent    rows of the recent window        -> n_recent_dev of the attention / layer calls
+ *   region_hi   first row of the recent window = end of the retrieval region
+ *                                                 -> dc_layer_args.region_hi_dev
+ *   append_pos  region_hi + n_recent             -> pos_dev of dc_append_kv_bf16 (with pos = 0)
+ *   overflow    set (and left set) when a step was counted although the window was full: that
+ *               token's row was not stored; the caller did not roll the window over in time
+ * dc_step_state_advance: n_recent = clamp(n_recent + delta, 0, limit), append_pos follows; once
+ * per decoded token, after the last layer (src/diffcache/kvcache/diffcache.py:221-223).
+ * dc_step_state_rollover: the oldest `moved` rows of the window join the region: region_hi +=
+ * moved, n_recent = keep, append_pos follows.  Stream-ordered, may sit between two replays of a
+ * captured step; the caller sketches the moved rows first (dc_sketch_build_bf16, keep_scale).
+ */
+typedef struct dc_step_state {
+    int32_t n_recent, region_hi, append_pos, overflow;
+} dc_step_state;
+int dc_step_state_advance(int32_t *state, int delta, int limit, void *stream);
+int dc_step_state_rollover(int32_t *state, int moved, int keep, void *stream);
+
+/*
  * Prefill ingest: src (n_b, seq, n_h, hd) -> store[b, h, dst_pos + s, :].
  * Replaces the permute(0,2,1,3).contiguous() + host copy + Index::prefill memcpy
  * (src/diffcache/kvcache/diffcache.py:142-147, diffcache_cpu/src/nsw.rs:503-508).
@@ -344,6 +367,13 @@ typedef struct dc_layer_args {
                              dc_gather_attn_bf16): n_recent is then its capacity */
     int one_kernel;       /* a DC_ONE_KERNEL_* value: when a short context may run as one kernel
                              (see "Short contexts" below); 0 = DC_ONE_KERNEL_AUTO */
+    const int32_t *region_hi_dev; /* NULL, or a device word holding the first row of the suffix
+                             (= the end of the retrieval region) at the time the kernels run;
+                             recent_lo is then its LARGEST value, which sizes the launches and the
+                             workspace, so that a call captured in a graph stays valid when the
+                             recent window is rolled over (dc_step_state).  Needs scores == NULL; the
+                             region must hold at least `budget` rows; takes the sketch or streaming
+                             route */
 } dc_layer_args;
 
 size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int group, int hd,

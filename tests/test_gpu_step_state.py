@@ -109,6 +109,124 @@ def test_decode_attention_captured_once_and_replayed_with_a_growing_window():
         (torch.randn(1000, device=DEV) * 2).sum().item()    # unrelated eager work between replays
 
 
+@pytest.mark.parametrize("with_sketch", [True, False])
+@pytest.mark.parametrize("order", [0, 1])
+def test_decode_layer_with_the_region_end_on_the_device(with_sketch, order):
+    """dc_layer_args.region_hi_dev through the C ABI: launches laid out for the largest region,
+    the live end read by the kernels.  For several live ends on ONE workspace (select state left
+    ready from call to call) the ids and the output equal those of a call that passes the same end
+    as a launch parameter."""
+    from diffcache_amd import _hip
+    rng = np.random.default_rng(75)
+    b, hkv, hq, hd, budget, p, n_max, cap_recent = 2, 2, 8, 128, 200, 4, 9000, 16
+    g = hq // hkv
+    k, v = rand_bf16(rng, b, hkv, n_max, hd), rand_bf16(rng, b, hkv, n_max, hd)
+    kd, vd = dev_bf16(k), dev_bf16(v)
+    hi_cap = n_max - cap_recent
+    sk = _hip.Sketch(kd).build(kd, p, hi_cap - p) if with_sketch else None
+    ws = _hip.alloc_workspace(_hip.layer_workspace_bytes(b * hkv, hi_cap - p, budget, g, hd, budget + p + cap_recent + 1), DEV)
+    state = torch.zeros((4,), dtype=torch.int32, device=DEV)
+    first = True
+    for hi, n_recent in [(2000, 5), (2001, 16), (8984, 0), (300, 7), (204, 16)]:
+        q = dev_bf16(rand_bf16(rng, b, hq, hd))
+        nk, nv = dev_bf16(rand_bf16(rng, b, hkv, hd)), dev_bf16(rand_bf16(rng, b, hkv, hd))
+        state.copy_(torch.tensor([n_recent, hi, hi + n_recent, 0], dtype=torch.int32))
+        idx_d = torch.full((b * hkv, budget), -1, dtype=torch.int32, device=DEV)
+        out_d = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+        print(f"region end on the device: hi={hi} n_recent={n_recent} sketch={with_sketch} order={order}", flush=True)
+        _hip.decode_layer(q, kd, vd, p, hi_cap, cap_recent, budget, None, idx_d, out_d, ws, nk, nv, order=order,
+                          select_state_ready=not first, sketch=sk, n_recent_dev=state[0:1], region_hi_dev=state[1:2])
+        assert _hip.last_route() == (_hip.ROUTE_SKETCH if with_sketch else _hip.ROUTE_STREAM)
+        first = False
+        idx_h = torch.full((b * hkv, budget), -1, dtype=torch.int32, device=DEV)
+        out_h = torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+        ws_h = _hip.alloc_workspace(_hip.layer_workspace_bytes(b * hkv, hi - p, budget, g, hd, budget + p + n_recent + 1), DEV)
+        _hip.decode_layer(q, kd, vd, p, hi, n_recent, budget, None, idx_h, out_h, ws_h, nk, nv, order=order,
+                          sketch=sk, one_kernel=_hip.ONE_KERNEL_NEVER)
+        torch.cuda.synchronize()
+        if order == _hip.ORDER_BEST:
+            assert torch.equal(idx_d, idx_h), (hi, n_recent)
+        else:
+            assert torch.equal(torch.sort(idx_d, dim=1).values, torch.sort(idx_h, dim=1).values), (hi, n_recent)
+        assert torch.allclose(out_d.float(), out_h.float(), atol=2e-3, rtol=2.0 ** -7), (hi, n_recent)
+
+
+@pytest.mark.parametrize("key_sketch", [True, False])
+def test_captured_step_survives_rollovers(key_sketch):
+    """Every layer's decode_attention captured ONCE; 3 x kvbuf_suffix_maxlen replays with
+    rollover() between them whenever the window is full.  The region's end, the window's length
+    and the append position are device words, so the one graph serves the whole generation (the
+    reference's graphs do: src/diffcache/base.py:46-55; its data layer takes every token:
+    diffcache_cpu/src/lib.rs:352-369).  Every step equals the eager call on a twin cache (which
+    rolls over by itself) and the oracle on the grown history."""
+    from diffcache_amd import _hip
+    rng = np.random.default_rng(74)
+    L, b, hkv, hq, hd, budget, p, s, smax, seq = 2, 2, 2, 8, 128, 96, 4, 6, 14, 1200
+    steps = 3 * smax
+    scale = np.exp(rng.standard_normal((1, 1, hkv, hd))).astype(np.float32)
+    K = [orc.f32_to_bf16(rng.standard_normal((b, seq, hkv, hd)).astype(np.float32) * scale) for _ in range(L)]
+    V = [rand_bf16(rng, b, seq, hkv, hd) for _ in range(L)]
+    caches = [make_cache(L, b, seq + steps + 8, hkv, hq, hd, budget, p, s, smax, key_sketch=key_sketch) for _ in range(3)]
+    for c in caches:
+        for l in range(L):
+            c.prefill_update_kv_cache(dev_bf16(K[l]), dev_bf16(V[l]), l)
+    graphed, eager, warm = caches
+    hist = History(K, V)
+    qs = [torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    nks = [torch.zeros((b, 1, hkv, hd), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    nvs = [torch.zeros((b, 1, hkv, hd), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    outs = [torch.zeros((b, hq, hd), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    for l in range(L):      # every kernel once outside capture (on the third cache)
+        warm.decode_attention(l, qs[l], nks[l], nvs[l], order=_hip.ORDER_BEST)
+    graphed._ensure_workspace()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for l in range(L):
+            graphed.decode_attention(l, qs[l], nks[l], nvs[l], out=outs[l], order=_hip.ORDER_BEST)
+    assert graphed.captured_region_on_device is True
+    want_suffix, rollovers, region0 = s, 0, graphed.retrieval_region_len
+    for step in range(steps):
+        if graphed.window_full():           # between two replays: stream-ordered, no capture again
+            assert graphed.rollover() == smax - s
+            want_suffix, rollovers = s, rollovers + 1
+        q_np = [rand_bf16(rng, b, hq, hd) for _ in range(L)]
+        big = 25.0 if step % 7 == 3 else 1.0    # some keys far outside the range the sketch was fitted to
+        nk_np = [rand_bf16(rng, b, 1, hkv, hd, scale=big) for _ in range(L)]
+        nv_np = [rand_bf16(rng, b, 1, hkv, hd) for _ in range(L)]
+        for l in range(L):
+            qs[l].copy_(dev_bf16(q_np[l]))
+            nks[l].copy_(dev_bf16(nk_np[l]))
+            nvs[l].copy_(dev_bf16(nv_np[l]))
+        print(f"replay {step}: region {graphed.retrieval_region_len} rows, window {want_suffix}", flush=True)
+        g.replay()
+        torch.cuda.synchronize()
+        assert graphed.retrieval_region_len == region0 + rollovers * (smax - s)
+        for l in range(L):
+            want = eager.decode_attention(l, qs[l], nks[l], nvs[l], order=_hip.ORDER_BEST)
+            torch.cuda.synchronize()
+            assert torch.equal(graphed.idx[l], eager.idx[l]), (step, l)
+            assert torch.equal(outs[l], want), (step, l)
+            check_against_oracle(graphed, hist, l, q_np[l], nk_np[l], nv_np[l], outs[l], graphed.idx[l], want_suffix)
+            hist.push(l, nk_np[l], nv_np[l])
+        graphed.advance_host_step()
+        want_suffix += 1
+        n_recent, region_hi, append_pos, overflow = graphed._state.tolist()
+        assert (n_recent, region_hi, append_pos, overflow) == (want_suffix, graphed._region()[1],
+                                                               graphed._region()[1] + want_suffix, 0)
+        assert eager.kvbuf_suffix_len == graphed.kvbuf_suffix_len and eager.generation == graphed.generation
+        (torch.randn(1000, device=DEV) * 2).sum().item()    # unrelated eager work between replays
+    assert rollovers >= 4
+    graphed.check_status()
+    # one replay too many without a rollover is not silent: the device notes the dropped token
+    while not graphed.window_full():
+        g.replay()
+        graphed.advance_host_step()
+    g.replay()
+    with pytest.raises(AssertionError, match="full recent window"):
+        graphed.check_status()
+
+
 @pytest.mark.parametrize("key_sketch", [True, False])
 def test_decode_attention_rolls_the_recent_window_over(key_sketch):
     """3 x kvbuf_suffix_maxlen decode steps: when the window is full its oldest rows join the
