@@ -36,13 +36,56 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one scan launch of configuration 3 moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
-# scaled by a known-size copy kernel: counts x 2 KiB read + counts x 1 KiB written.  Taken
-# once, when the profile summaries kept with this repository were made -- not in this run.
-SCAN_TRAFFIC_PROFILED_C3 = {"sketch": 524_698 * 2048 + 16_457 * 1024,
-                            "bf16": 1_048_497 * 2048 + 14_402 * 1024}
-# the one-kernel route of configuration 2 (small_layer_kernel), same counters
-LAYER_TRAFFIC_PROFILED_C2 = 35_234 * 2048 + 1_477 * 1024
+# HBM bytes per launch of the dominant kernels, from rocprofv3 FETCH_SIZE and WRITE_SIZE scaled by a
+# known-size copy kernel.  Taken when the profile summaries kept with this repository were made,
+# not in this run; the figures live in one file that the summaries quote as well.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def profiled_traffic(key: str):
+    """HBM bytes per launch of `key` ("c3.sketch", "c3.bf16", "c2.one_kernel") from the tracked
+    counter file, or None."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            e = json.load(f)["kernels"][key]
+        return int(e["fetch_counts"] * e["fetch_unit_bytes"] + e["write_counts"] * e["write_unit_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def device_state() -> dict:
+    """Clock levels, power and partition modes of the GPU as the driver's sysfs files report them
+    (plain file reads; whatever is missing or unreadable is left out).  Read before and after a
+    timed loop: the same binary has been seen at two speed levels of the scan on these boxes."""
+    import glob
+    out = {}
+    for card in sorted(glob.glob("/sys/class/drm/card[0-9]*/device")):
+        if not os.path.exists(os.path.join(card, "pp_dpm_sclk")) and \
+                not os.path.exists(os.path.join(card, "current_compute_partition")):
+            continue
+        st = {}
+        for name in ("pp_dpm_sclk", "pp_dpm_mclk", "pp_dpm_fclk", "pp_dpm_socclk", "current_compute_partition",
+                     "current_memory_partition", "power_dpm_force_performance_level", "gpu_busy_percent",
+                     "mem_busy_percent"):
+            try:
+                with open(os.path.join(card, name)) as f:
+                    txt = f.read().strip()
+            except OSError:
+                continue
+            if name.startswith("pp_dpm_"):      # keep the active level(s): the lines marked with '*'
+                act = [ln.strip() for ln in txt.splitlines() if ln.rstrip().endswith("*")]
+                txt = "; ".join(act) if act else txt.replace("\n", "; ")
+            st[name] = txt
+        for hw in glob.glob(os.path.join(card, "hwmon", "hwmon*")):
+            for name in ("power1_average", "power1_input", "temp1_input", "freq1_input", "freq2_input"):
+                try:
+                    with open(os.path.join(hw, name)) as f:
+                        st[name] = f.read().strip()
+                except OSError:
+                    pass
+        if st:
+            out[os.path.basename(os.path.dirname(card))] = st
+    return out
 
 CONFIGS = {
     # name: layers, batch, q heads, kv heads, hd, context, budget, sinks, recent
@@ -234,6 +277,7 @@ class DecodeWorkload:
             for _ in range(warmup):
                 step(None)
             torch.cuda.synchronize()
+            state_before = device_state()
             t0 = time.perf_counter()
             marks[0].record()
             for s in range(steps):
@@ -242,6 +286,7 @@ class DecodeWorkload:
                     marks[(s + 1) // group].record()
             torch.cuda.synchronize()
             elapsed = time.perf_counter() - t0
+        state_after = device_state()
         ms_per_step = elapsed * 1e3 / steps
         per_step_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 / group for i in range(n_marks))
 
@@ -320,14 +365,25 @@ class DecodeWorkload:
             "frac_8d": rows_bytes_8d / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         }
         one_kernel = kernel.startswith("small_layer_kernel")
-        if (self.name == "c3" and scan in SCAN_TRAFFIC_PROFILED_C3) or (self.name == "c2" and one_kernel):
-            roofline["traffic"] = LAYER_TRAFFIC_PROFILED_C2 if one_kernel else SCAN_TRAFFIC_PROFILED_C3[scan]
-            roofline["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE when the committed profile " \
-                                         "summaries were taken, not measured in this run"
+        key = "c2.one_kernel" if (self.name == "c2" and one_kernel) else f"{self.name}.{scan}"
+        roofline["traffic"] = profiled_traffic(key)
+        if roofline["traffic"] is not None:
+            roofline["traffic_source"] = "profiles/hbm_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE when " \
+                                         "the committed profile summaries were taken, not measured in this run"
+        # The same binary has been seen at two levels of the scan's speed (about +10 %), constant
+        # within a process: say which one this run was at (configuration 3 only, where it was seen).
+        level = None
+        if self.name == "c3" and not one_kernel and scan in ("sketch", "bf16"):
+            level = "fast" if scan_ms * 1e3 < (185.0 if scan == "sketch" else 342.0) else "slow"
         s_per_step = ms_per_step * 1e-3
         return {
             "value": ms_per_step * 1e3, "unit": "us", "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
             "workload": cfg["desc"], "scan": scan,
+            # the arithmetic the route computes in: the sketch scan reads one byte per key element
+            # and the rows that survive are rescored from the bf16 keys in fp32
+            "dtype": "bf16" if (one_kernel or scan != "sketch") else "u8 sketch scan + bf16 exact rescoring",
+            "level": level,
+            "device_state": {"before": state_before, "after": state_after},
             "call_path": call_path,
             "step_us_p10_p50_p90": [pct(0.10), pct(0.50), pct(0.90)],
             "roofline": roofline,
@@ -514,9 +570,11 @@ def main() -> int:
         out = dict(head)
         out.update({"value": res["value"], "unit": res["unit"], "steps": res["steps"], "warmup": res["warmup"],
                     "ms_per_step": res["ms_per_step"]})
+        if "dtype" in res:
+            out["dtype"] = res["dtype"]
         out["config"] = dict({"workload": res["workload"], "call_path": res["call_path"]}, **extra_config)
         for k, v in res.items():
-            if k not in ("value", "unit", "steps", "warmup", "ms_per_step", "workload", "call_path"):
+            if k not in ("value", "unit", "steps", "warmup", "ms_per_step", "workload", "call_path", "dtype"):
                 out[k] = v
         return out
 
