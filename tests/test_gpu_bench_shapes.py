@@ -110,6 +110,8 @@ def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units, mutate=None
         worst_lit = max(worst_lit, float(np.max(err[big] / np.abs(want[big]))))
     print(f"{cfg_name}: worst score error = {worst_bar:.3f} of the 1e-5*sum|q_i k_i| bar; "
           f"{worst_lit:.2e} relative to |s| (literal bar 1e-5, rows with |s| >= 1)", flush=True)
+    # the literal bar of the task: scores within 1e-5 relative (fp32), wherever |s| is not tiny
+    assert worst_lit <= 1e-5, (cfg_name, "scores, relative to |s|", worst_lit)
 
     # attention of a few units against the float64 softmax over the oracle's row set
     worst_abs, worst_small, worst_ulp = 0.0, 0.0, 0.0
@@ -133,6 +135,9 @@ def check_layer(cfg_name: str, cfg_id: int, attn_units, score_units, mutate=None
             worst_ulp = max(worst_ulp, float((err / ulp).max()))
     print(f"{cfg_name}: worst attention error = {worst_abs:.2e} absolute; {worst_small:.2e} where |out| < 0.5 "
           f"(literal bar 2e-3); {worst_ulp:.2f} bf16 ulps of the output (0.5 = correctly rounded)", flush=True)
+    # the literal bar of the task: 2e-3 absolute in bf16, wherever bf16 can hold a step of 2e-3
+    # (|out| < 0.5: one bf16 ulp is below 2e-3 there; larger values are held to |x| * 2^-8 above)
+    assert worst_small <= 2e-3, (cfg_name, "attention where |out| < 0.5", worst_small)
     return ids["dense"], sc
 
 

@@ -59,11 +59,15 @@ def test_static_scratch_attention_matches_the_workspace_entry_point():
         want = hip.gather_attn(q, k, v, idx, n_idx, lo, sink, hi, recent, nk, nv, lse=want_lse, n_idx_unit=n_unit)
         out = torch.full_like(want, float("nan"))
         lse = torch.full_like(want_lse, float("nan"))
+        torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
+        free_before = torch.cuda.mem_get_info()[0]          # the driver's count: sees a hipMalloc inside the library too
         rc = _static_call(hip, k, v, q, nk, nv, idx, n_unit, lo, hi, sink, recent, out, lse)
         assert rc == 0, hip.lib.dc_last_error().decode()
         assert torch.cuda.memory_allocated() == before
         torch.cuda.synchronize()
+        if case is not cases[0]:    # (the first call on a device resolves the array's address: the code object may be loaded then)
+            assert torch.cuda.mem_get_info()[0] == free_before, case
         assert torch.equal(out.view(torch.int16), want.view(torch.int16)), case
         assert torch.equal(lse, want_lse), case
 
