@@ -108,7 +108,9 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
         if (!ready) dc_ws_state_initialised(a->workspace);
     }
     g_last_route = k_eff <= 0 ? DC_ROUTE_ATTEND_ONLY
-                              : (a->scores ? DC_ROUTE_DENSE : (a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM));
+                              : (a->scores ? DC_ROUTE_DENSE
+                                           : (a->sketch_codes && region <= DC_SKETCH_MAX_ROWS ? DC_ROUTE_SKETCH
+                                                                                             : DC_ROUTE_STREAM));
     if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY && !a->region_hi_dev &&
         dc_small_supported(n_units, region, k_eff, a->group, a->hd)) {
         // short context: the whole layer in one kernel whose blocks are all resident (ids in no
@@ -132,7 +134,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
             return DC_OK;
         }
     }
-    if (k_eff > 0 && !a->scores && a->sketch_codes) {
+    if (k_eff > 0 && !a->scores && a->sketch_codes && region <= DC_SKETCH_MAX_ROWS) {
         // streaming select over the 8-bit sketch, exact rescoring of the kept rows
         DC_REQUIRE(a->sketch_scale && a->sketch_resid, "dc_decode_layer: sketch_scale / sketch_resid missing");
         rc = dc_sketch_select_impl(
@@ -192,7 +194,7 @@ extern "C" int dc_decode_layer_route(const dc_layer_args *a) {
     if (a->order == DC_ORDER_ANY && a->one_kernel != DC_ONE_KERNEL_NEVER && !a->region_hi_dev &&
         dc_small_supported(n_units, region, k_eff, a->group, a->hd))
         return DC_ROUTE_ONE_KERNEL;
-    return a->sketch_codes ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;
+    return a->sketch_codes && region <= DC_SKETCH_MAX_ROWS ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;
 }
 
 extern "C" int dc_decode_layer_status(const dc_layer_args *a, void *stream) {

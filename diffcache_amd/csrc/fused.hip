@@ -68,10 +68,10 @@ __device__ __forceinline__ void lds_store_relaxed(uint32_t *p, uint32_t v) {
 // the unit's list with one returning atomic, flush the block's histogram, and in
 // the blocks chosen by the caller refresh the unit's running threshold from
 // whatever part of the histogram is visible.  Staleness only loosens the bound.
-template <int kT = kThreads>
-__device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 *wstage, uint32_t wcnt,
+template <int kT = kThreads, typename E = uint2>
+__device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const E *wstage, uint32_t wcnt,
                                                    uint32_t *s_wcnt, uint32_t *s_base, uint32_t *wtot,
-                                                   UnitState *st, uint32_t *hu, uint2 *surv_unit,
+                                                   UnitState *st, uint32_t *hu, E *surv_unit,
                                                    bool refresh, uint32_t kk) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -92,7 +92,7 @@ __device__ __forceinline__ void prune_block_finish(uint32_t *lhist, const uint2 
     }
     __syncthreads();
     {
-        uint2 *dst = surv_unit + *s_base + wbase;
+        E *dst = surv_unit + *s_base + wbase;
         for (uint32_t i = lane; i < wcnt; i += 64) dst[i] = wstage[i];
     }
     if (!refresh) return;
@@ -259,7 +259,15 @@ __device__ __forceinline__ float sketch_dot16(const uint4 &c, const float (&w)[1
 // bucket(approx_i + margin) is not worse than the running threshold bucket,
 // margin = 2E' + Q.  The kept rows are rescored exactly by rescore_kernel.
 constexpr uint32_t kBulkKeep = 96;      // of the 128 rows of a wave's first two steps
-constexpr float kUnseenApprox = 3.0e38f;  // approximation of a row the scan did not read: better than any score
+// What the sketch scan keeps of a row: the row, and the bucket of (approximation + margin), which
+// is all the exact pass asks of it (the exact pass keeps the row when that bucket is not worse
+// than the final threshold bucket).  One word instead of (row, approximation): a byte the scan
+// writes costs it several bytes read.  Rows of a unit beyond 2^22 do not fit: the callers send
+// such regions down the bf16 route.
+constexpr int kSketchRowBits = 22;
+constexpr int kSketchMaxRows = 1 << kSketchRowBits;
+static_assert(kSketchMaxRows == DC_SKETCH_MAX_ROWS && DC_HIST_BINS <= (1 << (32 - kSketchRowBits)), "row and bucket share a word");
+__device__ __forceinline__ uint32_t sketch_entry(uint32_t bucket, uint32_t row) { return (bucket << kSketchRowBits) | row; }
 
 template <int HD, bool SHARED_POLL>
 __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kernel(
@@ -271,7 +279,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     constexpr int LPR = HD / 16;  // lanes per row, 16 code bytes each
     const int n_rows = dc_live_rows(n_cap, hi_dev, lo_row);
     __shared__ uint32_t lhist[DC_HIST_BINS];
-    __shared__ uint2 stage[kStage];
+    __shared__ uint32_t stage[kStage];  // kept rows as kSketchEntry words
     __shared__ uint32_t s_tb;  // the block's copy of the unit's running threshold bucket
     __shared__ uint32_t wtot[kThreads / 64 + 1];
     __shared__ uint32_t s_wcnt[kThreads / 64];
@@ -339,7 +347,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     if (tid == 0) s_tb = tb;
     __syncthreads();
 
-    uint2 *wstage = stage + wave * (kBigSteps * 64);
+    uint32_t *wstage = stage + wave * (kBigSteps * 64);
     uint32_t wcnt = 0, marginal = 0;
     const unsigned long long lt = (1ull << lane) - 1ull;
 
@@ -370,11 +378,11 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
         }
         const int64_t myrow = row0 + lane;
         const bool valid = myrow < n_rows;
-        const uint32_t lb = dc_score_bucket(mine);
-        const bool keep = valid && dc_score_bucket(mine + margin) <= tb;
+        const uint32_t lb = dc_score_bucket(mine), kb = dc_score_bucket(mine + margin);
+        const bool keep = valid && kb <= tb;
         if (keep) atomicAdd(&lhist[lb], 1u);
         const unsigned long long mask = __ballot(keep);
-        if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(mine));
+        if (keep) wstage[wcnt + __popcll(mask & lt)] = sketch_entry(kb, (uint32_t)myrow);
         wcnt += (uint32_t)__popcll(mask);
         if (decltype(count)::value) marginal += (uint32_t)__popcll(__ballot(keep && lb >= tb));
     };
@@ -438,15 +446,17 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
             const int64_t myrow = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64 + lane;
             const bool keep = myrow < n_rows;
             const unsigned long long mask = __ballot(keep);
-            if (keep) wstage[wcnt + __popcll(mask & lt)] = make_uint2((uint32_t)myrow, __float_as_uint(kUnseenApprox));
+            if (keep) wstage[wcnt + __popcll(mask & lt)] = sketch_entry(0u, (uint32_t)myrow);  // passes any threshold
             wcnt += (uint32_t)__popcll(mask);
         }
     } else if (step < my_steps) {
         work_step(step, ca, std::false_type{});  // an odd last step; its rows are already on the way
     }
     const bool refresh = small ? (chunk & 3) == 3 : ((chunk - small_chunks) & 7) == 7;
-    prune_block_finish(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st, hist + (int64_t)unit * DC_HIST_BINS,
-                       surv + (int64_t)unit * n_cap, refresh, (uint32_t)k_eff);
+    prune_block_finish<kThreads, uint32_t>(lhist, wstage, wcnt, s_wcnt, &s_base, wtot, st,
+                                           hist + (int64_t)unit * DC_HIST_BINS,
+                                           reinterpret_cast<uint32_t *>(surv) + (int64_t)unit * n_cap, refresh,
+                                           (uint32_t)k_eff);
 }
 
 // The same scan for the PQ baseline: a key's score is its ADC score (dc_pq.h), read
@@ -690,18 +700,17 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     auto entry = [&](uint32_t t) { return ((uint32_t)blk + t * (uint32_t)nblk) * kThreads + (uint32_t)tid; };
 
     // the block's first batch of the list is requested before the threshold is worked out
-    const uint2 *su = surv + (int64_t)unit * n_rows;
-    uint2 p[kRescoreBatch];
+    const uint32_t *su = reinterpret_cast<const uint32_t *>(surv) + (int64_t)unit * n_rows;
+    uint32_t p[kRescoreBatch];
 #pragma unroll
     for (int j = 0; j < kRescoreBatch; ++j) {
         const uint32_t i = entry((uint32_t)j);
-        p[j] = make_uint2(0u, 0u);
+        p[j] = 0xffffffffu;
         if ((uint32_t)j < my_tiles && i < n_s) p[j] = su[i];
     }
     uint32_t tb, c_less;
     unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
     if (blk == 0 && tid == 0) st->c_less = 0;
-    const float margin = __uint_as_float(st->margin);
     float q[8];
     dc_load_query<HD>(Q, unit, q_group, col, q);
     const uint16_t *Ku = K + b * sb + h * sh + col * 8;
@@ -716,16 +725,16 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
             const uint32_t i = entry(t);
             const bool in = t < my_tiles && i < n_s;
             if (t0 != 0) {
-                p[j] = make_uint2(0u, 0u);
+                p[j] = 0xffffffffu;
                 if (in) p[j] = su[i];
             }
-            if (in && dc_score_bucket(__uint_as_float(p[j].y) + margin) <= tb) pass |= 1u << j;
+            if (in && (p[j] >> kSketchRowBits) <= tb) pass |= 1u << j;
         }
         uint32_t n_c;
         uint32_t pos = block_excl_scan<kThreads>(__popc(pass), wtot, &n_c);
 #pragma unroll
         for (int j = 0; j < kRescoreBatch; ++j)
-            if (pass & (1u << j)) cid[pos++] = p[j].x;
+            if (pass & (1u << j)) cid[pos++] = p[j] & (uint32_t)(kSketchMaxRows - 1);
         // the list slot is reserved now and looked at after the rows are scored
         uint32_t base_reg = 0;
         if (tid == 0 && n_c) base_reg = atomicAdd(&st->cand_cnt, n_c);
@@ -1098,6 +1107,8 @@ int dc_sketch_scan_launch(const char *who, const void *k, const uint8_t *codes, 
                "%s: key strides must be multiples of 8 elements and row_stride >= hd", who);
     DC_REQUIRE(cb % 16 == 0 && ch % 16 == 0 && cr % 16 == 0 && cr >= hd,
                "%s: code strides must be multiples of 16 bytes and row_stride >= hd", who);
+    DC_REQUIRE(n_rows <= kSketchMaxRows, "%s: %d rows per unit; the sketch scan takes at most %d (use the bf16 scan)", who,
+               n_rows, kSketchMaxRows);
     FusedPlan p;
     int rc = plan_fused(who, n_b, n_h, n_rows, budget, &p);
     if (rc) return rc;

@@ -49,6 +49,7 @@ extern "C" {
 #define DC_EDEVICE (-6)   /* a kernel gave up a bounded wait: the outputs of that call are not valid */
 
 #define DC_HIST_BINS 1024 /* histogram bins per unit used by the select */
+#define DC_SKETCH_MAX_ROWS (1 << 22) /* rows of a unit the sketch scan takes (its lists name a row in 22 bits) */
 
 /* Library version (DC_VERSION).  Replaces nothing; added for binding checks. */
 int dc_version(void);
@@ -153,7 +154,8 @@ int dc_score_select_bf16(const void *k, const void *q, uint32_t *idx_out, int64_
  *     keep_scale != 0: the existing scales are used (values outside their range are
  *     clamped) and the residual bounds are raised where needed -- call it on rows
  *     appended later (replaces nothing in the reference; goes with lib.rs:352-369).
- *   dc_score_select_sketch_bf16   arguments as dc_score_select_bf16 plus the sketch;
+ *   dc_score_select_sketch_bf16   arguments as dc_score_select_bf16 plus the sketch; n_rows at most
+ *     DC_SKETCH_MAX_ROWS (dc_decode_layer streams the bf16 keys of a longer region instead);
  *     state_ready as in dc_layer_args.select_state_ready; the optional event pair is
  *     recorded around the scan of the codes.
  */
