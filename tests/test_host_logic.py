@@ -65,6 +65,53 @@ def test_one_kernel_guard_rule():
     assert _hip.last_route() == _hip.ROUTE_ATTEND_ONLY
 
 
+def test_route_of_a_region_too_long_for_the_sketch_scan():
+    """The sketch scan names a row in 22 bits; dc_decode_layer streams the bf16 keys of a longer
+    region instead (same ids).  dc_decode_layer_route follows no pointers, so it runs without a GPU."""
+    from diffcache_amd import _hip
+    a = _hip.LayerArgs()
+    a.n_b, a.n_h, a.group, a.hd, a.budget, a.n_sink = 1, 1, 4, 128, 64, 4
+    a.sketch_codes = 0x1000          # only looked at for "is there a sketch"
+    a.order = _hip.ORDER_BEST
+    a.recent_lo = 4 + (1 << 22)
+    assert _hip.lib.dc_decode_layer_route(ctypes.byref(a)) == _hip.ROUTE_SKETCH
+    a.recent_lo = 4 + (1 << 22) + 1
+    assert _hip.lib.dc_decode_layer_route(ctypes.byref(a)) == _hip.ROUTE_STREAM
+    a.sketch_codes = None
+    a.recent_lo = 5000
+    assert _hip.lib.dc_decode_layer_route(ctypes.byref(a)) == _hip.ROUTE_STREAM
+    a.budget = 0
+    assert _hip.lib.dc_decode_layer_route(ctypes.byref(a)) == _hip.ROUTE_ATTEND_ONLY
+
+
+def test_scan_kernels_do_not_spill():
+    """The scan kernels sit at the edge of their register budget (four waves per SIMD): a change
+    that makes the compiler spill costs them 10 us per launch without failing any parity test.
+    Compiles the file that holds them once more with the compiler's resource report."""
+    import shutil
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    src = os.path.join(ROOT, "diffcache_amd", "csrc", "fused.hip")
+    res = subprocess.run([hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "--cuda-device-only",
+                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-fast-math",
+                          "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", os.devnull],
+                         capture_output=True, text=True, cwd=os.path.dirname(src))
+    assert res.returncode == 0, res.stderr[-2000:]
+    name, seen, bad = None, 0, []
+    for line in res.stderr.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"VGPRs Spill: (\d+)", line)
+        if m and name and ("prune_kernel" in name or "rescore_kernel" in name):
+            seen += 1
+            if int(m.group(1)) > 0:
+                bad.append((name, int(m.group(1))))
+    assert seen >= 8, "the compiler's report was not understood"
+    assert not bad, bad
+
+
 def test_wrappers_refuse_cpu_tensors():
     from diffcache_amd import _hip
     k = torch.zeros((1, 1, 16, 128), dtype=torch.bfloat16)
