@@ -688,31 +688,33 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     const int tid = threadIdx.x;
     const int grp = tid / LPR, col = tid % LPR;
     UnitState *st = state + unit;
-    uint32_t n_s = st->surv_cnt;
-    if (n_s > (uint32_t)n_rows) n_s = n_rows;
     // The list is dealt to the unit's blocks in tiles of kThreads entries, round robin:
     // the scan appends in the order its blocks finish, and the entries of late blocks
     // (tight threshold) pass the filter far more often than those of early ones, so
     // contiguous slices would leave a few blocks with most of the gathers.
-    const uint32_t n_tiles = (n_s + kThreads - 1) / kThreads;
-    if ((uint32_t)blk >= n_tiles) return;
-    const uint32_t my_tiles = (n_tiles - (uint32_t)blk + (uint32_t)nblk - 1) / (uint32_t)nblk;
     auto entry = [&](uint32_t t) { return ((uint32_t)blk + t * (uint32_t)nblk) * kThreads + (uint32_t)tid; };
 
-    // the block's first batch of the list is requested before the threshold is worked out
+    // The block's first batch of the list is requested before its length is known (what lies
+    // beyond the length is stale and is masked below), together with the length, the histogram
+    // and the query: one memory round trip for all of them.
     const uint32_t *su = reinterpret_cast<const uint32_t *>(surv) + (int64_t)unit * n_rows;
     uint32_t p[kRescoreBatch];
 #pragma unroll
     for (int j = 0; j < kRescoreBatch; ++j) {
         const uint32_t i = entry((uint32_t)j);
         p[j] = 0xffffffffu;
-        if ((uint32_t)j < my_tiles && i < n_s) p[j] = su[i];
+        if (i < (uint32_t)n_rows) p[j] = su[i];
     }
-    uint32_t tb, c_less;
-    unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
-    if (blk == 0 && tid == 0) st->c_less = 0;
+    uint32_t n_s = st->surv_cnt;
     float q[8];
     dc_load_query<HD>(Q, unit, q_group, col, q);
+    uint32_t tb, c_less;
+    unit_threshold(hist + (int64_t)unit * DC_HIST_BINS, (uint32_t)k_eff, wtot, sres, tb, c_less);
+    if (n_s > (uint32_t)n_rows) n_s = n_rows;
+    const uint32_t n_tiles = (n_s + kThreads - 1) / kThreads;
+    if ((uint32_t)blk >= n_tiles) return;
+    const uint32_t my_tiles = (n_tiles - (uint32_t)blk + (uint32_t)nblk - 1) / (uint32_t)nblk;
+    if (blk == 0 && tid == 0) st->c_less = 0;
     const uint16_t *Ku = K + b * sb + h * sh + col * 8;
     uint32_t *ck = cand_key + (int64_t)unit * n_rows;
     uint32_t *ci = cand_idx + (int64_t)unit * n_rows;
