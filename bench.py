@@ -342,8 +342,8 @@ class DecodeWorkload:
         rows_bytes_8d = nu * self.region * hd * 2             # one launch, every bf16 key row once
         scan_bytes = rows_bytes_8d // 2 if scan == "sketch" else rows_bytes_8d + \
             (nu * self.region * 4 if scan == "dense" else 0)
-        kernel = {"sketch": "sketch_prune_kernel<128>", "bf16": "score_prune_kernel<128>",
-                  "dense": "score_kernel<128>"}[scan]
+        kernel = {"sketch": "sketch_prune_kernel", "bf16": "score_prune_kernel",
+                  "dense": "score_kernel"}[scan] + "<%d>" % hd
         call_path = "dc_decode_layer" + {"sketch": " (sketch scan + exact rescoring)", "bf16": "",
                                          "dense": " (dense scores)"}[scan]
         if self.layer(0, scan, mode, route_only=True) == self.hip.ROUTE_ONE_KERNEL:
@@ -531,6 +531,10 @@ def main() -> int:
     ap.add_argument("--stepwise", action="store_true",
                     help="config c4 only: the PQ search through the separate entry points (dense ADC "
                          "score array) instead of dc_pq_search_bf16")
+    ap.add_argument("--shape", default=None, metavar="KEY=VALUE,...",
+                    help="a decode step of another shape, timed like a single --config: any of layers, batch, "
+                         "hq, hkv, hd, ctx, budget, sink, recent (defaults: configuration 3 with 4 layers), "
+                         "e.g. --shape batch=2,ctx=524288.  Not a BASELINE configuration: no CPU leg")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one decode step (all layers) in a HIP graph and time its replays; "
                          "reported as graph_step_us (always done for configuration 2)")
@@ -539,6 +543,21 @@ def main() -> int:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
               "use --gpus 1", file=sys.stderr)
         return 2
+    if args.shape is not None:
+        cfg = dict(CONFIGS["c3"], id=6, layers=4)
+        try:
+            for item in args.shape.split(","):
+                key, val = item.split("=")
+                if key not in ("layers", "batch", "hq", "hkv", "hd", "ctx", "budget", "sink", "recent"):
+                    raise ValueError(key)
+                cfg[key] = int(val)
+        except ValueError as e:
+            print(f"bench.py: bad --shape ({e})", file=sys.stderr)
+            return 2
+        cfg["desc"] = ("other shape: {layers} layers, batch {batch}, ctx {ctx}, {hq}q/{hkv}kv heads, hd {hd}, "
+                       "top-k {budget} + {sink} sinks + {recent} recent".format(**cfg))
+        CONFIGS["shape"] = cfg
+        args.config, args.no_cpu = "shape", True
     if args.config == "all" and args.scan is not None:
         print("bench.py: --scan goes with a single --config", file=sys.stderr)
         return 2

@@ -357,7 +357,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     // compiler wait for exactly the older buffer instead of for every load in flight.
     const int64_t blk_end = block_row0 + (int64_t)steps * kRowsPerBlockStep - 1;
     const int64_t blk_last = blk_end < (int64_t)last ? blk_end : (int64_t)last;
-    auto load_step = [&](int step, uint4 (&cv)[LPR]) {
+    auto load_step = [&](int step, uint4 (&cv)[LPR]) __attribute__((always_inline)) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
 #pragma unroll
         for (int j = 0; j < LPR; ++j) {
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     };
     // COUNT: also count the rows kept although their own bucket is not better than the
     // threshold's (ties and near-ties); only the first two steps of a wave do.
-    auto work_step = [&](int step, const uint4 (&cv)[LPR], auto count) {
+    auto work_step = [&](int step, const uint4 (&cv)[LPR], auto count) __attribute__((always_inline)) {
         const int64_t row0 = block_row0 + (int64_t)step * kRowsPerBlockStep + wave * 64;
         float mine = 0.f;
 #pragma unroll
@@ -408,7 +408,7 @@ __global__ __launch_bounds__(kThreads, HD <= 128 ? 4 : 1) void sketch_prune_kern
     // polls and passes the value on through LDS.  With many units every wave polls for
     // itself, which keeps its threshold one step fresher.
     // (SHARED_POLL is a template parameter: as a run-time choice it costs registers.)
-    auto two_steps = [&](auto count) {
+    auto two_steps = [&](auto count) __attribute__((always_inline)) {
         uint32_t tb_next = tb;
         if (!SHARED_POLL || wave == 0) tb_next = load_relaxed(&st->tb_run);
         load_step(step + 1, cb2);

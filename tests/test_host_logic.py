@@ -86,8 +86,11 @@ def test_route_of_a_region_too_long_for_the_sketch_scan():
 
 def test_scan_kernels_do_not_spill():
     """The scan kernels sit at the edge of their register budget (four waves per SIMD): a change
-    that makes the compiler spill costs them 10 us per launch without failing any parity test.
-    Compiles the file that holds them once more with the compiler's resource report."""
+    that makes the compiler spill costs them 10 us per launch without failing any parity test, and
+    a lambda that the compiler declines to inline keeps the arrays it is handed in scratch memory
+    (no "spill" in the report, only a scratch size: the head-dim-256 sketch scan ran at a quarter
+    of its speed that way).  Compiles the file that holds them once more with the compiler's
+    resource report."""
     import shutil
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
@@ -103,12 +106,12 @@ def test_scan_kernels_do_not_spill():
         m = re.search(r"Function Name: (\S+)", line)
         if m:
             name = m.group(1)
-        m = re.search(r"VGPRs Spill: (\d+)", line)
+        m = re.search(r"(VGPRs Spill|ScratchSize \[bytes/lane\]): (\d+)", line)
         if m and name and ("prune_kernel" in name or "rescore_kernel" in name):
             seen += 1
-            if int(m.group(1)) > 0:
-                bad.append((name, int(m.group(1))))
-    assert seen >= 8, "the compiler's report was not understood"
+            if int(m.group(2)) > 0:
+                bad.append((name, m.group(1), int(m.group(2))))
+    assert seen >= 16, "the compiler's report was not understood"
     assert not bad, bad
 
 
