@@ -219,6 +219,9 @@ class DecodeWorkload:
         self.stream = torch.cuda.Stream(device=dev)     # default priority
         self.clean = False
         self.calls = {}
+        # this process has the GPU to itself and one stream: short contexts may run as one kernel
+        # inside the captured step as well (--one-kernel never: the kernel chain at any size)
+        self.one_kernel = hip.ONE_KERNEL_EXCLUSIVE
 
     def layer(self, l: int, scan: str, mode: int, ev=None, route_only: bool = False):
         """One dc_decode_layer call.  scan: "sketch", "bf16" or "dense" (fp32 scores +
@@ -234,9 +237,7 @@ class DecodeWorkload:
                 q, k, v, cfg["sink"], self.hi, cfg["recent"], cfg["budget"],
                 self.scores if scan == "dense" else None, self.idx, self.out, self.ws, nk, nv,
                 mode=mode, order=hip.ORDER_ANY, sketch=self.sketches[l] if scan == "sketch" else None,
-                # this process has the GPU to itself and one stream: short contexts may run as one
-                # kernel inside the captured step as well
-                one_kernel=hip.ONE_KERNEL_EXCLUSIVE)
+                one_kernel=self.one_kernel)
         if route_only:
             return call.route()
         call(select_state_ready=self.clean and scan != "dense", scan_events=ev)
@@ -535,6 +536,9 @@ def main() -> int:
                     help="a decode step of another shape, timed like a single --config: any of layers, batch, "
                          "hq, hkv, hd, ctx, budget, sink, recent (defaults: configuration 3 with 4 layers), "
                          "e.g. --shape batch=2,ctx=524288.  Not a BASELINE configuration: no CPU leg")
+    ap.add_argument("--one-kernel", default="exclusive", choices=["exclusive", "never"],
+                    help="single --config / --shape: never = take the kernel chain also where the context is "
+                         "short enough for the one-kernel route")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one decode step (all layers) in a HIP graph and time its replays; "
                          "reported as graph_step_us (always done for configuration 2)")
@@ -608,6 +612,8 @@ def main() -> int:
     if args.config != "all":
         scan = args.scan or "sketch"
         work = DecodeWorkload(torch, hip, args.config, dev, sketch=scan == "sketch")
+        if args.one_kernel == "never":
+            work.one_kernel = hip.ONE_KERNEL_NEVER
         res = work.measure(scan, mode, steps, warmup, args.event_stride, graph=args.graph or args.config == "c2",
                            cold=args.config == "c2")
         out = line(res, {"key_mode": args.mode})

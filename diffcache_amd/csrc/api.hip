@@ -112,7 +112,7 @@ extern "C" int dc_decode_layer(const dc_layer_args *a, void *stream) {
                                            : (a->sketch_codes && region <= DC_SKETCH_MAX_ROWS ? DC_ROUTE_SKETCH
                                                                                              : DC_ROUTE_STREAM));
     if (k_eff > 0 && !a->scores && a->order == DC_ORDER_ANY && !a->region_hi_dev &&
-        dc_small_supported(n_units, region, k_eff, a->group, a->hd)) {
+        dc_small_supported(n_units, region, k_eff, a->group, a->hd, a->sketch_codes != nullptr)) {
         // short context: the whole layer in one kernel whose blocks are all resident (ids in no
         // particular order); reads the bf16 keys, with or without a sketch.  The state is set up
         // for this route even when the call is sent down the chain below (another launch of the
@@ -192,7 +192,7 @@ extern "C" int dc_decode_layer_route(const dc_layer_args *a) {
     if (n_units == 0 || k_eff <= 0) return DC_ROUTE_ATTEND_ONLY;
     if (a->scores) return DC_ROUTE_DENSE;
     if (a->order == DC_ORDER_ANY && a->one_kernel != DC_ONE_KERNEL_NEVER && !a->region_hi_dev &&
-        dc_small_supported(n_units, region, k_eff, a->group, a->hd))
+        dc_small_supported(n_units, region, k_eff, a->group, a->hd, a->sketch_codes != nullptr))
         return DC_ROUTE_ONE_KERNEL;
     return a->sketch_codes && region <= DC_SKETCH_MAX_ROWS ? DC_ROUTE_SKETCH : DC_ROUTE_STREAM;
 }

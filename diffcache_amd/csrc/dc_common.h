@@ -59,7 +59,7 @@ int dc_gather_attn_common(const char *who, const void *q, const void *k, const v
                           int64_t ksh, int64_t ksr, int64_t vsb, int64_t vsh, int64_t vsr, float scale,
                           void *workspace, size_t workspace_bytes, void *stream, const int32_t *recent_lo_dev);
 // small.hip: a whole decode layer in one kernel, for short contexts
-bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd);
+bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd, bool has_sketch);
 size_t dc_small_workspace_bytes(int n_units, int region, int group, int hd);
 size_t dc_small_cand_bytes(int n_units, int region);
 int dc_small_state_init(int n_units, int region, void *cand, void *stream);

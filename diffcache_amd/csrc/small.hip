@@ -46,6 +46,9 @@ constexpr int kSmallRows = 4096;     // rows a block scores at most (their score
 constexpr int kSmallCand = 4096;     // candidates of a unit that are ranked in LDS
 constexpr int kSmallBlocks = 512;    // blocks of a launch at most: two per CU
 constexpr int64_t kSmallTotalRows = 640 * 1024;  // rows of all units that the route takes on (measured crossover)
+// ... and rows per unit when the caller brings a sketch (measured: 8 units, 43.3 us against 41.6 us
+// for the sketch chain at 49152 rows, 37.3 against 40.6 at 32768; 16 units: 53.4 against 50.8 at 40960)
+constexpr int kSmallSketchRows = 40 * 1024;
 constexpr int kSmallMl = 2048;       // floats of (m, l) the merge keeps in LDS: blocks per unit * G * 2
 
 struct SmallArgs {
@@ -896,7 +899,7 @@ void dc_ws_state_initialised(const void *workspace) {
 // Whether a layer of these sizes can take the one-kernel route: every block must be resident at
 // once (the blocks of a unit wait for each other), a block's rows must fit its LDS, and the
 // merge must hold the (m, l) pairs of a unit's blocks.
-bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd) {
+bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd, bool has_sketch) {
     // DIFFCACHE_ONE_KERNEL=0 in the environment (read once) switches the route off, for processes
     // that share the GPU with kernels that never leave their CUs
     static const bool enabled = [] {
@@ -907,6 +910,8 @@ bool dc_small_supported(int n_units, int region, int k_eff, int group, int hd) {
     if (k_eff < 1 || group < 1 || group > 8 || !(hd == 64 || hd == 128 || hd == 256)) return false;
     const SmallPlan p = plan_small(n_units, region);
     if (!p.ok || p.bpu * group * 2 > kSmallMl) return false;
+    // a caller with a sketch has the faster chain: there the kernel only wins up to 40 Ki rows per unit
+    if (has_sketch && region > kSmallSketchRows) return false;
     const int hi = hd == 64 ? 0 : (hd == 128 ? 1 : 2);
     const int dev = current_device();
     if (dev < 0) return false;

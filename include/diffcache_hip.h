@@ -383,7 +383,8 @@ size_t dc_layer_workspace_bytes(int n_units, int n_region_rows, int budget, int 
 int dc_decode_layer(const dc_layer_args *args, void *stream);
 /*
  * Short contexts.  With scores == NULL, order == DC_ORDER_ANY and at most 640 Ki region rows
- * over all units, dc_decode_layer runs the layer as ONE kernel whose blocks are all resident
+ * over all units (and, when a sketch is passed, whose chain of kernels is the faster one, at most
+ * 40 Ki region rows per unit), dc_decode_layer runs the layer as ONE kernel whose blocks are all resident
  * (two per CU) and hand their phases over through the workspace (same results; the event pair
  * then brackets that kernel).  No counterpart in the reference, whose layers run on the CPU pool
  * (lib.rs:352-369); what it has to match is that one layer call is always right

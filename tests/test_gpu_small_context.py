@@ -368,6 +368,33 @@ def test_prepared_layer_call_equals_decode_layer():
         assert torch.allclose(out[0].float(), out[1].float(), atol=2e-3, rtol=2.0 ** -7)
 
 
+def test_a_sketch_moves_the_crossover_to_the_chain():
+    """With a sketch the kernel chain is the faster one from about 40 Ki rows per unit on, so the
+    one-kernel route ends there; without a sketch it goes on to 640 Ki rows in all.  Both routes
+    select the same ids."""
+    torch.manual_seed(306)
+    b, hq, hkv, hd, budget = 1, 8, 2, 128, 512
+    for n_ctx, want_with_sketch in ((40 * 1024 + 68, hip.ROUTE_ONE_KERNEL), (40 * 1024 + 69, hip.ROUTE_SKETCH)):
+        kd = torch.randn((b, hkv, n_ctx, hd), device=DEV).to(torch.bfloat16)
+        vd = torch.randn((b, hkv, n_ctx, hd), device=DEV).to(torch.bfloat16)
+        qd = torch.randn((b, hq, hd), device=DEV).to(torch.bfloat16)
+        lo, hi, s_len = 4, n_ctx - 64, 64
+        sk = hip.Sketch(kd).build(kd, lo, hi - lo)
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, hi - lo, budget, hq // hkv, hd, budget + 69), DEV)
+        got = {}
+        for name, sketch in (("plain", None), ("sketch", sk)):
+            idx = torch.zeros((b * hkv, budget), dtype=torch.int32, device=DEV)
+            out = torch.empty((b, hq, hd), dtype=torch.bfloat16, device=DEV)
+            call = hip.LayerCall(qd, kd, vd, lo, hi, s_len, budget, None, idx, out, ws, sketch=sketch)
+            assert call.route() == (hip.ROUTE_ONE_KERNEL if sketch is None else want_with_sketch), (n_ctx, name)
+            call(select_state_ready=False)
+            torch.cuda.synchronize()
+            assert hip.last_route() == call.route()
+            got[name] = (torch.sort(idx, dim=1).values.cpu(), out.float().cpu())
+        assert torch.equal(got["plain"][0], got["sketch"][0]), n_ctx
+        assert torch.allclose(got["plain"][1], got["sketch"][1], atol=2e-3, rtol=2.0 ** -7), n_ctx
+
+
 def test_small_context_agrees_with_the_kernel_chain_on_random_cases():
     """120 random shapes, budgets, key modes and data laws: the one-kernel route (ids in any
     order) against the chain of kernels that the same call takes when the ids are asked best
