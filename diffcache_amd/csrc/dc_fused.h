@@ -10,7 +10,7 @@ constexpr int kRowsPerBlockStep = 256;
 constexpr int kBigSteps = 8;       // 2048 rows per large block
 constexpr int kSmallChunks = 16;   // leading 256-row blocks per unit
 constexpr int kStage = kBigSteps * kRowsPerBlockStep;
-constexpr int kCandLds = 8192;     // candidates the finish kernel keeps in LDS
+constexpr int kCandLds = 16384;    // candidates the finish kernel keeps in LDS (128 KB of the CU's 160)
 constexpr int kSharedPollUnits = 8;   // sketch scan: up to this many units, one wave per block polls
 constexpr int kPqThreads = 512;    // PQ scan: threads per block = keys per step
 constexpr int kPqBigSteps = 8;     // PQ scan: 4096 keys per large block

@@ -8,7 +8,7 @@ constexpr int kFinalThreads = 1024;
 constexpr int kRadixBits = 11;
 constexpr int kRadixBins = 1 << kRadixBits;
 constexpr int kScanBatch = 8;  // items of a list that a thread fetches before it looks at any
-constexpr int kScanShort = 8192;  // lists up to this length sit in LDS (kCandLds of the callers): plain loops
+constexpr int kScanShort = 8192;  // lists in global memory up to this length are read with plain loops
 
 // inclusive scan over the lanes of a wave: four shifts inside the rows of 16 lanes, then the
 // last lane of row 0 (2) is added to row 1 (3), and the last lane of row 1 to rows 2 and 3
@@ -60,9 +60,9 @@ __device__ __forceinline__ uint32_t wave_reserve(bool want, uint32_t *counter) {
 
 // f(key, id, valid) for every entry of a (key, id) list, by ALL threads the same number of times
 // (valid: the thread has an entry this time), so that f may use wave-wide operations.
-template <int NT, typename F>
+template <int NT, bool IN_LDS = false, typename F>
 __device__ __forceinline__ void dc_for_each_pair_uniform(const uint32_t *ck, const uint32_t *ci, uint32_t n, F f) {
-    if (n <= (uint32_t)kScanShort) {
+    if (IN_LDS || n <= (uint32_t)kScanShort) {
         for (uint32_t i0 = 0; i0 < n; i0 += NT) {
             const uint32_t i = i0 + threadIdx.x;
             const bool in = i < n;
@@ -114,7 +114,7 @@ __device__ __forceinline__ void dc_for_each_pair(const uint32_t *ck, const uint3
 // `prefix`, histogram bits [top-1, top-width) and find the bin that holds the
 // rem-th smallest (1-based).  Updates prefix (bin bits filled in), rem (rank inside
 // the bin), eq (bin size) and top (= the lowest decided bit).  Uniform over the block.
-template <typename Get>
+template <bool IN_LDS = false, typename Get>
 __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &prefix, uint32_t &rem,
                                                  uint32_t &eq, int &top, uint32_t *lh, uint32_t *wtot,
                                                  uint32_t *sres) {
@@ -124,7 +124,8 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
     for (int i = tid; i < kRadixBins; i += kFinalThreads) lh[i] = 0;
     __syncthreads();
     const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
-    if (n <= (uint32_t)kScanShort) {  // a list that the caller keeps in LDS: nothing to hide
+    constexpr bool kPlain = IN_LDS;  // a list that the caller keeps in LDS: nothing to hide
+    if (kPlain || n <= (uint32_t)kScanShort) {
         for (uint32_t i = tid; i < n; i += kFinalThreads) {
             uint32_t v;
             if (get(i, &v) && ((v & himask) == (prefix & himask)))
@@ -134,7 +135,7 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
     // kScanBatch items of a thread are fetched before any is looked at: with one load per
     // iteration a long list costs a memory round trip per item and thread.  A wave whose lanes
     // all hit one bin (long runs of equal keys) adds its count once.
-    for (uint32_t i0 = tid; n > (uint32_t)kScanShort && i0 < n; i0 += kScanBatch * kFinalThreads) {
+    for (uint32_t i0 = tid; !kPlain && n > (uint32_t)kScanShort && i0 < n; i0 += kScanBatch * kFinalThreads) {
         uint32_t v[kScanBatch];
         bool in[kScanBatch];
 #pragma unroll
@@ -187,11 +188,11 @@ __device__ __forceinline__ void block_radix_pass(Get get, uint32_t n, uint32_t &
 // subset.  get(i, &value) returns false for items outside the subset.  Returns the
 // threshold value; *rem_out = how many items equal to it are needed (rank of the
 // threshold inside its tie group), *n_eq = size of the tie group.
-template <typename Get>
+template <bool IN_LDS = false, typename Get>
 __device__ __forceinline__ uint32_t block_radix_select(Get get, uint32_t n, uint32_t rem, int top, uint32_t prefix,
                                        uint32_t eq, uint32_t *lh, uint32_t *wtot, uint32_t *sres,
                                        uint32_t *rem_out, uint32_t *n_eq) {
-    while (top > 0) block_radix_pass(get, n, prefix, rem, eq, top, lh, wtot, sres);
+    while (top > 0) block_radix_pass<IN_LDS>(get, n, prefix, rem, eq, top, lh, wtot, sres);
     *rem_out = rem;
     *n_eq = eq;
     return prefix;
@@ -201,7 +202,9 @@ __device__ __forceinline__ uint32_t block_radix_select(Get get, uint32_t n, uint
 // their ids to io[0, need).  Must be called by all kFinalThreads threads of a
 // block with uniform arguments.  lh: kRadixBins words, wtot: kFinalThreads/64+1
 // words, sres: 4 words, smisc: 2 words of LDS.  kout (optional) receives the
-// key of each id written.
+// key of each id written.  IN_LDS: ck and ci point into LDS (any length); lists in global
+// memory longer than kScanShort are read kScanBatch entries per thread at a time.
+template <bool IN_LDS = false>
 __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint32_t *ci, uint32_t n_c, uint32_t need,
                                  uint32_t *io, int n_rows, uint32_t *lh, uint32_t *wtot,
                                  uint32_t *sres, uint32_t *smisc, uint32_t *kout = nullptr) {
@@ -222,9 +225,10 @@ __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint3
     __syncthreads();
     const uint32_t k0 = ck[0];
     uint32_t diff = 0;
-    if (n_c <= (uint32_t)kScanShort)
+    const bool plain = IN_LDS || n_c <= (uint32_t)kScanShort;
+    if (plain)
         for (uint32_t i = tid; i < n_c; i += kFinalThreads) diff |= ck[i] ^ k0;
-    for (uint32_t i0 = tid; n_c > (uint32_t)kScanShort && i0 < n_c; i0 += kScanBatch * kFinalThreads) {
+    for (uint32_t i0 = tid; !plain && i0 < n_c; i0 += kScanBatch * kFinalThreads) {
         uint32_t v[kScanBatch];
 #pragma unroll
         for (int u = 0; u < kScanBatch; ++u) {
@@ -248,7 +252,7 @@ __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint3
         *v = ck[i];
         return true;
     };
-    if (top > 0) block_radix_pass(get_key, n_c, prefix, rem, eq, top, lh, wtot, sres);
+    if (top > 0) block_radix_pass<IN_LDS>(get_key, n_c, prefix, rem, eq, top, lh, wtot, sres);
 
     if (eq <= (uint32_t)kFinalThreads) {
         // The keys whose decided bits equal the threshold bin's are few: they are
@@ -260,7 +264,7 @@ __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint3
         __syncthreads();
         const uint32_t himask = (top >= 32) ? 0u : (0xffffffffu << top);
         const uint32_t base = need - rem;  // members from the bins below the threshold bin
-        dc_for_each_pair_uniform<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
+        dc_for_each_pair_uniform<kFinalThreads, IN_LDS>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
             const uint32_t hi = key & himask, ph = prefix & himask;
             const bool member = in && hi < ph, tied = in && hi == ph;
             const uint32_t slot = wave_reserve(member, &smisc[1]);
@@ -287,7 +291,7 @@ __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint3
 
     uint32_t need_eq, n_eq;
     const uint32_t t_key =
-        block_radix_select(get_key, n_c, rem, top, prefix, eq, lh, wtot, sres, &need_eq, &n_eq);
+        block_radix_select<IN_LDS>(get_key, n_c, rem, top, prefix, eq, lh, wtot, sres, &need_eq, &n_eq);
 
     uint32_t t_idx = 0xffffffffu;
     if (need_eq < n_eq) {  // only the lowest ids of the tie group fit
@@ -298,10 +302,10 @@ __device__ __forceinline__ void dc_finalize_unit(const uint32_t *ck, const uint3
             return ck[i] == t_key;
         };
         uint32_t r2, e2;
-        t_idx = block_radix_select(get_idx, n_c, need_eq, hbi + 1, 0u, n_eq, lh, wtot, sres, &r2, &e2);
+        t_idx = block_radix_select<IN_LDS>(get_idx, n_c, need_eq, hbi + 1, 0u, n_eq, lh, wtot, sres, &r2, &e2);
     }
 
-    dc_for_each_pair_uniform<kFinalThreads>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
+    dc_for_each_pair_uniform<kFinalThreads, IN_LDS>(ck, ci, n_c, [&](uint32_t key, uint32_t id, bool in) {
         const bool member = in && (key < t_key || (key == t_key && id <= t_idx));
         const uint32_t slot = wave_reserve(member, &smisc[1]);
         if (member && slot < need) {

@@ -906,7 +906,7 @@ __global__ __launch_bounds__(kFinalThreads) void select_finish_kernel(
     // Two calls, so that the staged list is read with LDS instructions: through a pointer chosen
     // at run time every access would be a flat one, and waiting for a flat load also waits for
     // the stores issued above.
-    if (staged) dc_finalize_unit(lck, lci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc, ko ? ko + c_less : nullptr);
+    if (staged) dc_finalize_unit<true>(lck, lci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc, ko ? ko + c_less : nullptr);
     else dc_finalize_unit(ck, ci, n_c, need, io + c_less, n_rows, lh, wtot, sres, smisc, ko ? ko + c_less : nullptr);
 }
 
