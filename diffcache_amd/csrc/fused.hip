@@ -688,6 +688,8 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
     const int tid = threadIdx.x;
     const int grp = tid / LPR, col = tid % LPR;
     UnitState *st = state + unit;
+    uint32_t opaque_zero = 0;
+    asm volatile("" : "+v"(opaque_zero));
     // The list is dealt to the unit's blocks in tiles of kThreads entries, round robin:
     // the scan appends in the order its blocks finish, and the entries of late blocks
     // (tight threshold) pass the filter far more often than those of early ones, so
@@ -737,9 +739,12 @@ __global__ __launch_bounds__(kThreads) void rescore_kernel(
 #pragma unroll
         for (int j = 0; j < kRescoreBatch; ++j)
             if (pass & (1u << j)) cid[pos++] = p[j] & (uint32_t)(kSketchMaxRows - 1);
-        // the list slot is reserved now and looked at after the rows are scored
+        // The list slot is reserved now and looked at after the rows are scored.  (Through an address
+        // the compiler cannot prove uniform: it turns an atomic on a uniform address into one atomic
+        // per wave plus a broadcast of the result and waits for that on the spot, a memory round
+        // trip in front of the barrier below and of every row request behind it.)
         uint32_t base_reg = 0;
-        if (tid == 0 && n_c) base_reg = atomicAdd(&st->cand_cnt, n_c);
+        if (tid == 0 && n_c) base_reg = atomicAdd(&st->cand_cnt + opaque_zero, n_c);
         __syncthreads();
         // exact scores: one LPR-lane group per row, kRowsInFlight rows of a group in flight
         constexpr int kRowsInFlight = 8;
