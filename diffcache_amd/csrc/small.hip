@@ -275,9 +275,22 @@ __global__ __launch_bounds__(kThreads) void small_layer_kernel(SmallArgs a) {
     // What an addition returns -- the rows of that bucket counted before this block's -- is the
     // block's place among the unit's rows of the bucket: every selected id and every candidate
     // gets its slot from the histogram, and no other counter is needed.
-    for (int i = tid; i < DC_HIST_BINS; i += kThreads) {
-        const uint32_t c = lhist[i];
-        lbase[i] = c ? atomicAdd(&hu[i], c) : 0u;
+    // (All of a thread's additions are issued before the first result is looked at: written as one
+    // loop over the bins the compiler waits for each addition before it issues the next, a memory
+    // round trip per bin and thread on the unit's critical path.)
+    {
+        constexpr int kPer = DC_HIST_BINS / kThreads;
+        static_assert(kPer * kThreads == DC_HIST_BINS, "bins per thread");
+        uint32_t before[kPer];
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const int i = tid + u * kThreads;
+            const uint32_t c = lhist[i];
+            before[u] = 0u;
+            if (c) before[u] = atomicAdd(&hu[i], c);
+        }
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) lbase[tid + u * kThreads] = before[u];
     }
 
     // ---------------- 2: threshold bucket; ids of better buckets, candidates of the threshold bucket ----------------
