@@ -37,7 +37,11 @@ __global__ __launch_bounds__(kThreads) void gather_attn_kernel(AttnArgs a) {
 template <int HD>
 __global__ __launch_bounds__(kThreads) void gather_attn_mfma_kernel(AttnArgs a, int group) {
     extern __shared__ float s_dyn[];
-    dc_attn_split_mfma<HD>(a, group, blockIdx.x / a.n_splits, blockIdx.x % a.n_splits, s_dyn);
+    // Split-major: a grid a little larger than what the device holds at once (config 3: 1088
+    // blocks on 1024 places) then ends on every unit's last, partial split instead of on the last
+    // units' full ones.
+    const int n_units = (int)(gridDim.x / (unsigned)a.n_splits);
+    dc_attn_split_mfma<HD>(a, group, blockIdx.x % n_units, blockIdx.x / n_units, s_dyn);
 }
 
 // out[u, g, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m): one block
