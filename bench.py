@@ -77,7 +77,9 @@ def device_state() -> dict:
                 txt = "; ".join(act) if act else txt.replace("\n", "; ")
             st[name] = txt
         for hw in glob.glob(os.path.join(card, "hwmon", "hwmon*")):
-            for name in ("power1_average", "power1_input", "temp1_input", "freq1_input", "freq2_input"):
+            # temp2: junction, temp3: memory (millidegrees), as their *_label files say on these boxes
+            for name in ("power1_average", "power1_input", "power1_cap", "temp1_input", "temp2_input", "temp3_input",
+                         "freq1_input", "freq2_input"):
                 try:
                     with open(os.path.join(hw, name)) as f:
                         st[name] = f.read().strip()
