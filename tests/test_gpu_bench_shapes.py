@@ -205,3 +205,27 @@ def test_config4_pq_search_full_size():
         # the exact scores themselves: float64 dot of the bf16 values
         want = orc.scores_f64(u16(q[u]), u16(store[u // index.h, u % index.h][torch.from_numpy(ws).to(DEV)]))
         assert np.max(np.abs(ex - want)) <= 1e-5 * np.max(np.abs(want)) + 1e-4
+
+
+def test_bench_line_of_another_shape():
+    """`bench.py --shape`: one JSON line with the contract's keys, on the chain and (same shape,
+    shorter context) on the one-kernel route."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for shape, scan, path in (("batch=2,ctx=49152,layers=2,budget=512", "sketch", "sketch scan"),
+                              ("batch=2,ctx=49152,layers=2,budget=512", "bf16", "dc_decode_layer"),
+                              ("batch=1,ctx=8192,layers=2,budget=256", "sketch", "one kernel")):
+        res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--shape", shape, "--scan", scan,
+                              "--steps", "3", "--warmup", "1"], capture_output=True, text=True, timeout=110)
+        assert res.returncode == 0, res.stderr[-2000:]
+        line = json.loads([ln for ln in res.stdout.splitlines() if ln.startswith("{")][-1])
+        for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+                    "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+            assert key in line, key
+        assert line["n_gpus"] == 1 and line["steps"] == 3 and line["value"] > 0 and line["cpu_baseline"] is None
+        assert path in line["config"]["call_path"], line["config"]
+        rf = line["roofline"]
+        assert rf["bound"] == "hbm" and 0 < rf["frac"] < 1 and rf["peak"] == 8000.0

@@ -240,6 +240,12 @@ def test_bench_refuses_more_than_one_gpu():
     assert res.returncode != 0 and "one GPU" in res.stderr
 
 
+def test_bench_refuses_an_unknown_shape_key():
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--shape", "batch=2,rows=5"],
+                         capture_output=True, text=True)
+    assert res.returncode != 0 and "bad --shape" in res.stderr
+
+
 # ---------------------------------------------------------------- snapshot codec
 
 def test_varint_known_answers():
