@@ -350,7 +350,8 @@ typedef struct dc_layer_args {
     int n_sink, n_recent; /* rows [0,n_sink) and [recent_lo, recent_lo+n_recent) always kept */
     int budget;           /* k */
     int mode, order;
-    float scale;          /* softmax scale, 1/sqrt(hd) in the reference */
+    float scale;          /* softmax scale, 1/sqrt(hd) in the reference (of the TRUE head dim when the rows
+                             are zero-padded to a supported one) */
     int select_state_ready; /* streaming select only (scores == NULL).  0: the workspace is
                              initialised first.  1: the caller vouches that the last call on this
                              workspace was a dc_decode_layer with the same n_b, n_h, group, hd,

@@ -395,6 +395,54 @@ def test_a_sketch_moves_the_crossover_to_the_chain():
         assert torch.allclose(got["plain"][1], got["sketch"][1], atol=2e-3, rtol=2.0 ** -7), n_ctx
 
 
+@pytest.mark.parametrize("hd", [96, 80, 192])
+def test_other_head_dims_run_zero_padded(hd):
+    """Head dims between the supported ones: rows, queries and values zero-padded to the next
+    supported size (a row stride of that size) and the softmax scale of the TRUE head dim give
+    the ids and the attention of the unpadded problem on every route; the padded output columns
+    come back zero."""
+    rng = np.random.default_rng(400 + hd)
+    pad = 128 if hd <= 128 else 256
+    b, hq, hkv, budget, mode = 1, 8, 2, 300, 0
+    g = hq // hkv
+    for n_ctx, with_sketch, order, want_route in ((5000, False, hip.ORDER_ANY, hip.ROUTE_ONE_KERNEL),
+                                                  (45000, True, hip.ORDER_ANY, hip.ROUTE_SKETCH),
+                                                  (45000, False, hip.ORDER_BEST, hip.ROUTE_STREAM)):
+        k, v, q = rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hkv, n_ctx, hd), rand_bf16(rng, b, hq, hd)
+        nk, nv = rand_bf16(rng, b, hkv, hd), rand_bf16(rng, b, hkv, hd)
+
+        def padded(a):
+            out = np.zeros(a.shape[:-1] + (pad,), dtype=np.uint16)
+            out[..., :hd] = a
+            return to_dev_bf16(out)
+
+        kd, vd, qd, nkd, nvd = padded(k), padded(v), padded(q), padded(nk), padded(nv)
+        p_len, s_len, lo, hi = orc.region_split(n_ctx, 4, 64)
+        region = hi - lo
+        sk = hip.Sketch(kd).build(kd, lo, region) if with_sketch else None
+        ws = hip.alloc_workspace(hip.layer_workspace_bytes(b * hkv, region, budget, g, pad, budget + 69), DEV)
+        idx = torch.full((b * hkv, budget), -1, dtype=torch.int32, device=DEV)
+        out = torch.full((b, hq, pad), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hip.decode_layer(qd, kd, vd, p_len, hi, s_len, budget, None, idx, out, ws, nkd, nvd, mode=mode,
+                         order=order, scale=1.0 / float(np.sqrt(hd)), sketch=sk)
+        torch.cuda.synchronize()
+        assert hip.last_route() == want_route, (hd, n_ctx)
+        dense = hip.score(kd, qd, lo, region, mode, q_group=g).cpu().numpy()
+        ids = idx.cpu().numpy().astype(np.int64)
+        got = orc.bf16_to_f32(to_np_u16(out))
+        assert not np.any(got[..., hd:]), hd
+        for u in range(b * hkv):
+            want = orc.topk_select(dense[u], budget, mode).astype(np.int64)
+            assert np.array_equal(np.sort(ids[u]), np.sort(want)), (hd, n_ctx, u)
+            # the scores of the padded rows are those of the unpadded ones (zeros add nothing)
+            exact = orc.bf16_to_f32(k[0, u, lo:hi]).astype(np.float64) @ \
+                orc.bf16_to_f32(orc.group_mean_bf16(q, hkv)[0, u]).astype(np.float64)
+            assert np.all(np.abs(dense[u] - exact) <= 1e-5 * np.maximum(1.0, np.abs(exact)) + 1e-4), (hd, u)
+            rows = np.concatenate([want + lo, np.arange(p_len), np.arange(hi, hi + s_len)]).astype(np.int64)
+            o, _ = orc.sparse_attention(q[0, u * g:(u + 1) * g], k[0, u][rows], v[0, u][rows], nk[0, u], nv[0, u])
+            assert bf16_close(got[0, u * g:(u + 1) * g, :hd], o), (hd, n_ctx, u)
+
+
 def test_small_context_agrees_with_the_kernel_chain_on_random_cases():
     """120 random shapes, budgets, key modes and data laws: the one-kernel route (ids in any
     order) against the chain of kernels that the same call takes when the ids are asked best
