@@ -207,6 +207,27 @@ def test_config4_pq_search_full_size():
         assert np.max(np.abs(ex - want)) <= 1e-5 * np.max(np.abs(want)) + 1e-4
 
 
+@pytest.mark.parametrize("name,over", [
+    ("batch1", dict(batch=1)),                                  # 8 units: short-scan grid, 1024-block exact pass
+    ("batch3", dict(batch=3)),                                  # 24 units x 131004 rows: just above 3 Mi rows in all
+    ("batch4_ctx32k", dict(batch=4, ctx=32768)),                # 32 units x 32700 rows
+    ("hd256", dict(batch=4, hkv=4, hq=16, hd=256, ctx=65536)),  # 16 units, head dim 256
+    ("hd64", dict(batch=2, hd=64, ctx=65536)),                  # 16 units, head dim 64
+])
+def test_other_shapes_all_routes(name, over):
+    """Shapes between the benchmark's configurations, where the grids of the scan and of the exact
+    pass are sized by other rules than at config 3: ids of all units on the three routes, scores
+    and attention of a few units (config 3's data law)."""
+    cfg = dict(bench.CONFIGS["c3"], id=6, layers=1)
+    cfg.update(over)
+    bench.CONFIGS["t_" + name] = cfg
+    try:
+        n_units = cfg["batch"] * cfg["hkv"]
+        check_layer("t_" + name, 6, attn_units=[0, n_units - 1], score_units=[0, n_units // 2])
+    finally:
+        del bench.CONFIGS["t_" + name]
+
+
 def test_bench_line_of_another_shape():
     """`bench.py --shape`: one JSON line with the contract's keys, on the chain and (same shape,
     shorter context) on the one-kernel route."""
