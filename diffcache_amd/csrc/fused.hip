@@ -1050,8 +1050,12 @@ int launch_select(const char *who, const FusedWs &w, uint32_t *idx_out, int64_t 
     uint32_t *sel_keys = order == DC_ORDER_BEST ? w.sel_keys : nullptr;
     // blocks per unit for the classify pass: one per 4096 rows of context, as long as
     // the grid stays near 2048 blocks
-    int nblk = (n_rows + 4095) / 4096;
-    const int cap = n_units >= 2048 ? 1 : 2048 / n_units;
+    // one block per 4096 rows and at most 2048 blocks; below 3 Mi rows in all, one per 1024 rows
+    // and at most 1024 blocks (8 x 131072 rows: 5.5 us against 7.1 us)
+    const bool few = (int64_t)n_units * n_rows < (3ll << 20);
+    int nblk = few ? (n_rows + 1023) / 1024 : (n_rows + 4095) / 4096;
+    const int grid = few ? 1024 : 2048;
+    const int cap = n_units >= grid ? 1 : grid / n_units;
     if (nblk > cap) nblk = cap;
     if (nblk < 1) nblk = 1;
     hipLaunchKernelGGL(classify_kernel, dim3((unsigned)n_units * (unsigned)nblk), dim3(kThreads), 0, st,
