@@ -1009,7 +1009,9 @@ int dc_score_prune_launch(const void *k, const void *q, int n_b, int n_h, int n_
     DC_REQUIRE(sb % 8 == 0 && sh % 8 == 0 && sr % 8 == 0 && sr >= hd,
                "dc_score_prune_bf16: strides must be multiples of 8 elements and row_stride >= hd");
     FusedPlan p;
-    int rc = plan_fused("dc_score_prune_bf16", n_b, n_h, n_rows, budget, &p);
+    // (short scans of up to 32 units: eight steps per block down to 512 blocks, like the sketch scan)
+    int rc = plan_fused("dc_score_prune_bf16", n_b, n_h, n_rows, budget, &p, kBigSteps, kRowsPerBlockStep,
+                        (int64_t)n_b * n_h <= 32 ? kSketchFillBlocks : 2048);
     if (rc) return rc;
     if (p.n_units == 0 || p.k_eff == 0) return DC_OK;
     FusedWs w;
